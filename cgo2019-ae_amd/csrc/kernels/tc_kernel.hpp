@@ -1,0 +1,380 @@
+// Device-side building blocks of the gfx950 tensor-contraction engine.
+//
+// The emitter writes, per contraction expression, a small configuration struct
+// (`Cfg`) and instantiates the templates below with it.  They take the place of
+// the CUDA kernel text the reference generator writes out
+// (cogent/src/codes/kernels/tc_code_kernel.py:20-135: shared-memory slices of
+// both inputs, a per-thread register tile, a K loop of {load, sync, outer
+// product, sync}, then the store), re-designed for CDNA4:
+//
+//   * one wavefront = 64 lanes; a block is WY x WX wavefronts;
+//   * the inner product runs on the matrix cores (v_mfma_f64_16x16x4_f64,
+//     v_mfma_f32_16x16x4_f32 or v_mfma_f32_32x32x2_f32); every wavefront owns
+//     TY x TX accumulator tiles;
+//   * the output tile is READ into the accumulators before the K loop, so the
+//     kernel computes C <- C +/- sum(A*B) (the reference kernel overwrites C,
+//     cogent/src/codes/kernels/tc_code_kernel_store_output.py:78) and the C
+//     loads overlap the staging of the first input slices;
+//   * both input slices are staged global -> registers -> LDS in the operand's
+//     own memory order (coalesced along its fastest index) and scattered into
+//     an LDS layout chosen per operand so that MFMA operand reads are
+//     bank-conflict free:
+//        LAY 0  "k-major"  addr = k * LD + e   (operand fastest index external)
+//        LAY 1  "e-major"  addr = e * LD + k   (operand fastest index contracted)
+//
+// Naming: the "X side" is the input that holds the output's fastest index; its
+// external indices run along the MFMA column (lane % 16) so that stores to C
+// are contiguous.  The "Y side" is the other input.  Composite coordinates:
+// x = x0 + tx0*(x1 + tx1*(...)) over the X-side external tiles, likewise y, k.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cogent {
+
+constexpr int TC_MAXI = 12;   // most distinct indices in one expression
+
+// Run-time geometry handed to every kernel (by value, in kernel-argument space).
+struct TcDims {
+    int ext[TC_MAXI];    // extent of every index id
+    int nblk[TC_MAXI];   // tiles along the index (grid factor for externals, K blocks for contracted)
+    int sC[TC_MAXI];     // element stride inside C  (0 when the index is absent)
+    int sX[TC_MAXI];     // element stride inside the X-side operand
+    int sY[TC_MAXI];     // element stride inside the Y-side operand
+    int nkb;             // number of K blocks = product of nblk over contracted ids
+    unsigned nblocks;    // number of output tiles = grid size
+};
+
+typedef double v4f64 __attribute__((ext_vector_type(4)));
+typedef float  v4f32 __attribute__((ext_vector_type(4)));
+typedef float  v16f32 __attribute__((ext_vector_type(16)));
+
+// Matrix-instruction traits.  Lane l of a wavefront supplies A[i = l % MT][k = l / MT]
+// and B[k = l / MT][j = l % MT]; row() gives the D row held in accumulator register r.
+template <int MI> struct Mfma;
+template <> struct Mfma<0> {   // v_mfma_f64_16x16x4_f64
+    typedef double T; typedef v4f64 Acc;
+    static constexpr int MT = 16, KSTEP = 4, NREG = 4;
+    __device__ static __forceinline__ int row(int r, int lane) { return 4 * r + lane / 16; }
+    __device__ static __forceinline__ Acc mma(T a, T b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+};
+template <> struct Mfma<1> {   // v_mfma_f32_16x16x4_f32
+    typedef float T; typedef v4f32 Acc;
+    static constexpr int MT = 16, KSTEP = 4, NREG = 4;
+    __device__ static __forceinline__ int row(int r, int lane) { return 4 * (lane / 16) + r; }
+    __device__ static __forceinline__ Acc mma(T a, T b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+};
+template <> struct Mfma<2> {   // v_mfma_f32_32x32x2_f32
+    typedef float T; typedef v16f32 Acc;
+    static constexpr int MT = 32, KSTEP = 2, NREG = 16;
+    __device__ static __forceinline__ int row(int r, int lane) { return 8 * (r / 4) + 4 * (lane / 32) + (r % 4); }
+    __device__ static __forceinline__ Acc mma(T a, T b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+};
+
+// View of one input operand of a Cfg (SIDE 0 = X, 1 = Y).
+template <class Cfg, int SIDE> struct Operand;
+template <class Cfg> struct Operand<Cfg, 0> {
+    static constexpr int R = Cfg::XR, LAY = Cfg::LAYX, LD = Cfg::LDX, BE = Cfg::BX, BEP = Cfg::BXP;
+    __device__ static __forceinline__ constexpr int id(int j)   { return Cfg::xo_id(j); }
+    __device__ static __forceinline__ constexpr int tile(int j) { return Cfg::xo_tile(j); }
+    __device__ static __forceinline__ constexpr int isk(int j)  { return Cfg::xo_isk(j); }
+    __device__ static __forceinline__ constexpr int mul(int j)  { return Cfg::xo_mul(j); }
+    __device__ static __forceinline__ int stride(const TcDims& d, int id) { return d.sX[id]; }
+};
+template <class Cfg> struct Operand<Cfg, 1> {
+    static constexpr int R = Cfg::YR, LAY = Cfg::LAYY, LD = Cfg::LDY, BE = Cfg::BY, BEP = Cfg::BYP;
+    __device__ static __forceinline__ constexpr int id(int j)   { return Cfg::yo_id(j); }
+    __device__ static __forceinline__ constexpr int tile(int j) { return Cfg::yo_tile(j); }
+    __device__ static __forceinline__ constexpr int isk(int j)  { return Cfg::yo_isk(j); }
+    __device__ static __forceinline__ constexpr int mul(int j)  { return Cfg::yo_mul(j); }
+    __device__ static __forceinline__ int stride(const TcDims& d, int id) { return d.sY[id]; }
+};
+
+template <class Op, int BKP>
+constexpr int lds_elems() { return Op::LAY == 0 ? BKP * Op::LD : Op::BEP * Op::LD; }
+
+template <class Op>
+__device__ __forceinline__ int lds_addr(int k, int e) { return Op::LAY == 0 ? k * Op::LD + e : e * Op::LD + k; }
+
+// Element q of an operand's slice, enumerated in the operand's memory order
+// (fastest index first, each index restricted to its tile): gives the element
+// offset relative to the slice origin, the LDS address and whether the element
+// lies inside the tensor.  rem[id] = extent[id] - tile origin along id.
+template <class Op, bool EXT_FULL, bool INT_FULL>
+__device__ __forceinline__ void slice_element(unsigned q, const TcDims& d, const int* rem,
+                                              int& goff, int& loff, bool& valid)
+{
+    int e = 0, k = 0;
+    goff = 0;
+    valid = true;
+#pragma unroll
+    for (int j = 0; j < Op::R; j++) {
+        const unsigned t = (unsigned)Op::tile(j);
+        const int i = (int)(q % t);
+        q /= t;
+        const int id = Op::id(j);
+        goff += i * Op::stride(d, id);
+        if (Op::isk(j)) {
+            k += i * Op::mul(j);
+            if (!INT_FULL) valid = valid && (i < rem[id]);
+        } else {
+            e += i * Op::mul(j);
+            if (!EXT_FULL) valid = valid && (i < rem[id]);
+        }
+    }
+    loff = lds_addr<Op>(k, e);
+}
+
+template <class Cfg, class Op, bool EXT_FULL, bool INT_FULL, int SLOTS>
+__device__ __forceinline__ void slice_load(typename Cfg::T (&reg)[SLOTS], const typename Cfg::T* __restrict__ src,
+                                           const TcDims& d, const int* rem, int tid)
+{
+    typedef typename Cfg::T T;
+    constexpr unsigned E = (unsigned)(Cfg::BK * Op::BE);
+#pragma unroll
+    for (int s = 0; s < SLOTS; s++) {
+        const unsigned q = (unsigned)tid + (unsigned)s * Cfg::NT;
+        int goff, loff; bool valid;
+        slice_element<Op, EXT_FULL, INT_FULL>(q, d, rem, goff, loff, valid);
+        T v = (T)0;
+        if ((E % Cfg::NT == 0 || q < E) && valid) v = src[goff];
+        reg[s] = v;
+    }
+}
+
+template <class Cfg, class Op, bool NEGATE, int SLOTS>
+__device__ __forceinline__ void slice_store(const typename Cfg::T (&reg)[SLOTS], typename Cfg::T* lds,
+                                            const TcDims& d, int tid)
+{
+    constexpr unsigned E = (unsigned)(Cfg::BK * Op::BE);
+#pragma unroll
+    for (int s = 0; s < SLOTS; s++) {
+        const unsigned q = (unsigned)tid + (unsigned)s * Cfg::NT;
+        int goff, loff; bool valid;
+        slice_element<Op, true, true>(q, d, nullptr, goff, loff, valid);
+        if (E % Cfg::NT == 0 || q < E) lds[loff] = NEGATE ? -reg[s] : reg[s];
+    }
+}
+
+// The contraction kernel.  EXT_FULL: every external extent is a multiple of its
+// tile and the tile products need no padding; INT_FULL: the same for the
+// contracted indices.  (The reference picks among four kernels by the same two
+// tests, cogent/src/codes/kernels/tc_interface.py:1150-1175.)
+template <class Cfg, bool EXT_FULL, bool INT_FULL>
+__global__ __launch_bounds__(Cfg::NT)
+void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __restrict__ X,
+                    const typename Cfg::T* __restrict__ Y, const TcDims d)
+{
+    typedef typename Cfg::T T;
+    typedef Mfma<Cfg::MI> MM;
+    typedef typename MM::Acc Acc;
+    typedef Operand<Cfg, 0> OX;
+    typedef Operand<Cfg, 1> OY;
+    constexpr int MT = MM::MT, NREG = MM::NREG, KSTEP = MM::KSTEP;
+    constexpr int TX = Cfg::TX, TY = Cfg::TY, NT = Cfg::NT;
+    constexpr int SLOTS_X = (Cfg::BK * Cfg::BX + NT - 1) / NT;
+    constexpr int SLOTS_Y = (Cfg::BK * Cfg::BY + NT - 1) / NT;
+    constexpr int LDS_X = lds_elems<OX, Cfg::BKP>();
+    constexpr int LDS_Y = lds_elems<OY, Cfg::BKP>();
+    constexpr bool PADDED = (Cfg::BKP != Cfg::BK) || (Cfg::BXP != Cfg::BX) || (Cfg::BYP != Cfg::BY);
+
+    __shared__ T lds_x[LDS_X];
+    __shared__ T lds_y[LDS_Y];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wx = wave % Cfg::WX;
+    const int wy = wave / Cfg::WX;
+
+    // ---- which output tile: X-side tiles vary fastest over the grid
+    int rem[Cfg::NIDX];
+    int64_t baseC = 0, baseX = 0, baseY = 0;
+    {
+        unsigned b = blockIdx.x;
+#pragma unroll
+        for (int i = 0; i < Cfg::NX; i++) {
+            const int id = Cfg::x_id(i);
+            const unsigned nb = (unsigned)d.nblk[id];
+            const int o = (int)(b % nb) * Cfg::x_tile(i);
+            b /= nb;
+            rem[id] = d.ext[id] - o;
+            baseC += (int64_t)o * d.sC[id];
+            baseX += (int64_t)o * d.sX[id];
+        }
+#pragma unroll
+        for (int i = 0; i < Cfg::NY; i++) {
+            const int id = Cfg::y_id(i);
+            const unsigned nb = (unsigned)d.nblk[id];
+            const int o = (int)(b % nb) * Cfg::y_tile(i);
+            b /= nb;
+            rem[id] = d.ext[id] - o;
+            baseC += (int64_t)o * d.sC[id];
+            baseY += (int64_t)o * d.sY[id];
+        }
+#pragma unroll
+        for (int i = 0; i < Cfg::NK; i++) rem[Cfg::k_id(i)] = d.ext[Cfg::k_id(i)];
+    }
+    T* __restrict__ Cb = C + baseC;
+    const T* __restrict__ Xb = X + baseX;
+    const T* __restrict__ Yb = Y + baseY;
+
+    // ---- where this lane's accumulator elements live in C (-1: outside)
+    int cx[TX];
+    int cy[TY][NREG];
+#pragma unroll
+    for (int tj = 0; tj < TX; tj++) {
+        const int x = (wx * TX + tj) * MT + lane % MT;
+        unsigned q = (unsigned)x;
+        int off = 0; bool ok = (Cfg::BXP == Cfg::BX) || (x < Cfg::BX);
+#pragma unroll
+        for (int i = 0; i < Cfg::NX; i++) {
+            const int c = (int)(q % (unsigned)Cfg::x_tile(i));
+            q /= (unsigned)Cfg::x_tile(i);
+            off += c * d.sC[Cfg::x_id(i)];
+            if (!EXT_FULL) ok = ok && (c < rem[Cfg::x_id(i)]);
+        }
+        cx[tj] = ok ? off : -1;
+    }
+#pragma unroll
+    for (int ti = 0; ti < TY; ti++) {
+#pragma unroll
+        for (int r = 0; r < NREG; r++) {
+            const int y = (wy * TY + ti) * MT + MM::row(r, lane);
+            unsigned q = (unsigned)y;
+            int off = 0; bool ok = (Cfg::BYP == Cfg::BY) || (y < Cfg::BY);
+#pragma unroll
+            for (int i = 0; i < Cfg::NY; i++) {
+                const int c = (int)(q % (unsigned)Cfg::y_tile(i));
+                q /= (unsigned)Cfg::y_tile(i);
+                off += c * d.sC[Cfg::y_id(i)];
+                if (!EXT_FULL) ok = ok && (c < rem[Cfg::y_id(i)]);
+            }
+            cy[ti][r] = ok ? off : -1;
+        }
+    }
+
+    // ---- accumulators start from the C tile: C_in + sum, summed in k order
+    Acc acc[TY][TX];
+#pragma unroll
+    for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+        for (int tj = 0; tj < TX; tj++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++) {
+                T v = (T)0;
+                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) v = Cb[cx[tj] + cy[ti][r]];
+                acc[ti][tj][r] = v;
+            }
+
+    // ---- padding rows/columns of the LDS slices are never written by the staging: clear once
+    if (PADDED) {
+        for (int i = tid; i < LDS_X; i += NT) lds_x[i] = (T)0;
+        for (int i = tid; i < LDS_Y; i += NT) lds_y[i] = (T)0;
+    }
+
+    // ---- K loop
+    int kbc[Cfg::NK > 0 ? Cfg::NK : 1];
+#pragma unroll
+    for (int i = 0; i < Cfg::NK; i++) kbc[i] = 0;
+
+    T rx[SLOTS_X], ry[SLOTS_Y];
+    slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb, d, rem, tid);
+    slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb, d, rem, tid);
+
+    for (int kb = 0; kb < d.nkb; kb++) {
+        __syncthreads();                       // previous slice fully consumed (and padding cleared)
+        slice_store<Cfg, OX, false>(rx, lds_x, d, tid);
+        slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y, d, tid);
+        __syncthreads();
+
+        if (kb + 1 < d.nkb) {
+            // advance the K-block odometer (first composite K index fastest) and prefetch
+            int64_t kx = 0, ky = 0;
+            bool carry = true;
+#pragma unroll
+            for (int i = 0; i < Cfg::NK; i++) {
+                const int id = Cfg::k_id(i);
+                if (carry) { kbc[i]++; carry = false; if (kbc[i] == d.nblk[id]) { kbc[i] = 0; carry = true; } }
+                const int o = kbc[i] * Cfg::k_tile(i);
+                rem[id] = d.ext[id] - o;
+                kx += (int64_t)o * d.sX[id];
+                ky += (int64_t)o * d.sY[id];
+            }
+            slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb + kx, d, rem, tid);
+            slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb + ky, d, rem, tid);
+        }
+
+#pragma unroll
+        for (int k4 = 0; k4 < Cfg::BKP / KSTEP; k4++) {
+            const int kk = k4 * KSTEP + lane / MT;
+            T a[TY], b[TX];
+#pragma unroll
+            for (int ti = 0; ti < TY; ti++) a[ti] = lds_y[lds_addr<OY>(kk, (wy * TY + ti) * MT + lane % MT)];
+#pragma unroll
+            for (int tj = 0; tj < TX; tj++) b[tj] = lds_x[lds_addr<OX>(kk, (wx * TX + tj) * MT + lane % MT)];
+#pragma unroll
+            for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+                for (int tj = 0; tj < TX; tj++) acc[ti][tj] = MM::mma(a[ti], b[tj], acc[ti][tj]);
+        }
+    }
+
+    // ---- write the tile back
+#pragma unroll
+    for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+        for (int tj = 0; tj < TX; tj++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++)
+                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) Cb[cx[tj] + cy[ti][r]] = acc[ti][tj][r];
+}
+
+// ---------------------------------------------------------------------------
+// Plain kernel: one lane per output element, contracted indices walked in
+// sum() order with separately rounded multiply and add, i.e. the summation
+// order of the reference's host check (cogent/drivers/tccg/code_main_tccg_01.c:117-133).
+// Used as the fallback for shapes the tiled kernel does not cover and as an
+// on-device cross-check of it.
+struct TcPlainDims {
+    int n_out, n_int;
+    int ext_out[TC_MAXI], sA_out[TC_MAXI], sB_out[TC_MAXI];
+    int ext_k[TC_MAXI], sA_k[TC_MAXI], sB_k[TC_MAXI];
+    int sign;
+    long long total;    // elements of C
+    long long ktotal;   // product of contracted extents
+};
+
+__device__ __forceinline__ double tc_mul_rn(double a, double b) { return __dmul_rn(a, b); }
+__device__ __forceinline__ float  tc_mul_rn(float a, float b)   { return __fmul_rn(a, b); }
+__device__ __forceinline__ double tc_add_rn(double a, double b) { return __dadd_rn(a, b); }
+__device__ __forceinline__ float  tc_add_rn(float a, float b)   { return __fadd_rn(a, b); }
+
+template <class T>
+__global__ __launch_bounds__(256)
+void tc_plain_kernel(T* __restrict__ C, const T* __restrict__ A, const T* __restrict__ B, const TcPlainDims p)
+{
+    const long long lin = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (lin >= p.total) return;
+    long long r = lin;
+    long long oa = 0, ob = 0;
+    for (int i = 0; i < p.n_out; i++) {
+        const int e = (int)(r % p.ext_out[i]);
+        r /= p.ext_out[i];
+        oa += (long long)e * p.sA_out[i];
+        ob += (long long)e * p.sB_out[i];
+    }
+    T acc = C[lin];
+    int k[TC_MAXI];
+    for (int i = 0; i < p.n_int; i++) k[i] = 0;
+    for (long long kk = 0; kk < p.ktotal; kk++) {
+        long long ka = oa, kb = ob;
+        for (int i = 0; i < p.n_int; i++) { ka += (long long)k[i] * p.sA_k[i]; kb += (long long)k[i] * p.sB_k[i]; }
+        const T prod = tc_mul_rn(A[ka], B[kb]);
+        acc = tc_add_rn(acc, p.sign < 0 ? -prod : prod);
+        for (int j = p.n_int - 1; j >= 0; j--) { if (++k[j] < p.ext_k[j]) break; k[j] = 0; }
+    }
+    C[lin] = acc;
+}
+
+}  // namespace cogent

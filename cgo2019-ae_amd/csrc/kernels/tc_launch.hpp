@@ -1,0 +1,176 @@
+// Host-side launch wrapper instantiated once per emitted expression.
+//
+// Takes the place of the host caller the reference generator writes out
+// (`sd_t_d2_fusion`, cogent/src/codes/kernels/tc_interface.py:10-101: grid
+// size, strides, the four-way full/partial kernel choice).  Differences, on
+// purpose: the pointers are DEVICE pointers and nothing is allocated or copied
+// here; every argument is validated and a status code is returned instead of
+// running unchecked; C is read-modify-written.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+#include "tc_kernel.hpp"
+
+namespace cogent {
+
+enum TcStatus {
+    TC_OK = 0,
+    TC_ERR_NULL_POINTER = 1,
+    TC_ERR_NEGATIVE_EXTENT = 2,
+    TC_ERR_TOO_LARGE = 3,      // a tensor has 2^31 or more elements, or the grid does not fit
+    TC_ERR_LAUNCH = 4,         // the HIP runtime refused the launch
+    TC_ERR_BAD_VARIANT = 5,
+    TC_ERR_ALLOC = 6,          // host-pointer shim only
+};
+
+inline char* tc_error_buffer() { static thread_local char buf[256] = ""; return buf; }
+inline int tc_fail(int code, const char* msg)
+{
+    snprintf(tc_error_buffer(), 256, "%s", msg);
+    return code;
+}
+// The runtime's "last error" is sticky per thread and may have been left by an unrelated earlier
+// call (an event query that was not ready, for instance): clear it before a launch, read it after.
+inline void tc_clear_hip_error() { (void)hipGetLastError(); }
+inline int tc_check_launch(const char* what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return TC_OK;
+    snprintf(tc_error_buffer(), 256, "%s: %s", what, hipGetErrorString(e));
+    return TC_ERR_LAUNCH;
+}
+
+enum TcVariant { TC_VARIANT_AUTO = 0, TC_VARIANT_PLAIN = 1, TC_VARIANT_TILED = 2 };
+
+// sizes[] holds one extent per index id: output indices in output order, then
+// the contracted indices in sum() order -- the order of the entry point's
+// `int size_*` parameters (cogent/src/codes/kernels/tc_interface.py:1459-1492).
+template <class Cfg>
+int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t stream, int variant)
+{
+    typedef typename Cfg::T T;
+    tc_error_buffer()[0] = 0;
+    if (variant < 0 || variant > 2) return tc_fail(TC_ERR_BAD_VARIANT, "unknown kernel variant");
+    for (int i = 0; i < Cfg::NIDX; i++)
+        if (sizes[i] < 0) return tc_fail(TC_ERR_NEGATIVE_EXTENT, "negative extent");
+    // empty output or empty sum: C is left as it is
+    for (int i = 0; i < Cfg::NIDX; i++)
+        if (sizes[i] == 0) return TC_OK;
+    if (!C || !A || !B) return tc_fail(TC_ERR_NULL_POINTER, "null tensor pointer");
+
+    // element strides: dense, first listed index fastest
+    int64_t sC[TC_MAXI] = {0}, sA[TC_MAXI] = {0}, sB[TC_MAXI] = {0};
+    int64_t nC = 1, nA = 1, nB = 1;
+    for (int j = 0; j < Cfg::CR; j++) { sC[Cfg::c_id(j)] = nC; nC *= sizes[Cfg::c_id(j)]; }
+    for (int j = 0; j < Cfg::AR; j++) { sA[Cfg::a_id(j)] = nA; nA *= sizes[Cfg::a_id(j)]; }
+    for (int j = 0; j < Cfg::BR; j++) { sB[Cfg::b_id(j)] = nB; nB *= sizes[Cfg::b_id(j)]; }
+    const int64_t lim = ((int64_t)1 << 31) - 1;
+    if (nC > lim || nA > lim || nB > lim) return tc_fail(TC_ERR_TOO_LARGE, "a tensor has more than 2^31-1 elements");
+
+    if (variant == TC_VARIANT_PLAIN) {
+        TcPlainDims p;
+        memset(&p, 0, sizeof(p));
+        p.n_out = Cfg::CR;
+        p.n_int = Cfg::NK;
+        p.total = nC;
+        p.ktotal = 1;
+        p.sign = Cfg::SIGN;
+        for (int j = 0; j < Cfg::CR; j++) {
+            const int id = Cfg::c_id(j);
+            p.ext_out[j] = sizes[id]; p.sA_out[j] = (int)sA[id]; p.sB_out[j] = (int)sB[id];
+        }
+        for (int j = 0; j < Cfg::NK; j++) {
+            const int id = Cfg::sum_id(j);
+            p.ext_k[j] = sizes[id]; p.sA_k[j] = (int)sA[id]; p.sB_k[j] = (int)sB[id];
+            p.ktotal *= sizes[id];
+        }
+        const int64_t grid = (nC + 255) / 256;
+        if (grid > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
+        tc_clear_hip_error();
+        hipLaunchKernelGGL(tc_plain_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream,
+                           (T*)C, (const T*)A, (const T*)B, p);
+        return tc_check_launch("plain kernel launch failed");
+    }
+
+    TcDims d;
+    memset(&d, 0, sizeof(d));
+    const int64_t* sX = Cfg::X_IS_A ? sA : sB;
+    const int64_t* sY = Cfg::X_IS_A ? sB : sA;
+    for (int i = 0; i < Cfg::NIDX; i++) {
+        d.ext[i] = sizes[i]; d.nblk[i] = 1;
+        d.sC[i] = (int)sC[i]; d.sX[i] = (int)sX[i]; d.sY[i] = (int)sY[i];
+    }
+    bool ext_full = (Cfg::BX == Cfg::BXP) && (Cfg::BY == Cfg::BYP);
+    bool int_full = (Cfg::BK == Cfg::BKP);
+    int64_t grid = 1;
+    for (int i = 0; i < Cfg::NX; i++) {
+        const int id = Cfg::x_id(i), t = Cfg::x_tile(i);
+        d.nblk[id] = (sizes[id] + t - 1) / t; grid *= d.nblk[id];
+        if (sizes[id] % t) ext_full = false;
+    }
+    for (int i = 0; i < Cfg::NY; i++) {
+        const int id = Cfg::y_id(i), t = Cfg::y_tile(i);
+        d.nblk[id] = (sizes[id] + t - 1) / t; grid *= d.nblk[id];
+        if (sizes[id] % t) ext_full = false;
+    }
+    int64_t nkb = 1;
+    for (int i = 0; i < Cfg::NK; i++) {
+        const int id = Cfg::k_id(i), t = Cfg::k_tile(i);
+        d.nblk[id] = (sizes[id] + t - 1) / t; nkb *= d.nblk[id];
+        if (sizes[id] % t) int_full = false;
+    }
+    if (grid > lim || nkb > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
+    d.nkb = (int)nkb;
+    d.nblocks = (unsigned)grid;
+
+    T* c = (T*)C;
+    const T* x = (const T*)(Cfg::X_IS_A ? A : B);
+    const T* y = (const T*)(Cfg::X_IS_A ? B : A);
+    const dim3 g((unsigned)grid), b(Cfg::NT);
+    tc_clear_hip_error();
+    if (ext_full && int_full)       hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true>),   g, b, 0, stream, c, x, y, d);
+    else if (ext_full)              hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false>),  g, b, 0, stream, c, x, y, d);
+    else if (int_full)              hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true>),  g, b, 0, stream, c, x, y, d);
+    else                            hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false>), g, b, 0, stream, c, x, y, d);
+    return tc_check_launch("tiled kernel launch failed");
+}
+
+// The reference's calling convention: HOST pointers in, result copied back
+// (cogent/src/codes/others/tc_pre_CUDA_Malloc.py:6-47 and
+// cogent/src/codes/kernels/tc_interface.py:1368-1419).  Off the timed path.
+template <class Cfg>
+int tc_run_host(const int* sizes, void* hC, const void* hA, const void* hB)
+{
+    typedef typename Cfg::T T;
+    for (int i = 0; i < Cfg::NIDX; i++)
+        if (sizes[i] < 0) return tc_fail(TC_ERR_NEGATIVE_EXTENT, "negative extent");
+    for (int i = 0; i < Cfg::NIDX; i++)
+        if (sizes[i] == 0) return TC_OK;
+    if (!hC || !hA || !hB) return tc_fail(TC_ERR_NULL_POINTER, "null tensor pointer");
+    int64_t nC = 1, nA = 1, nB = 1;
+    for (int j = 0; j < Cfg::CR; j++) nC *= sizes[Cfg::c_id(j)];
+    for (int j = 0; j < Cfg::AR; j++) nA *= sizes[Cfg::a_id(j)];
+    for (int j = 0; j < Cfg::BR; j++) nB *= sizes[Cfg::b_id(j)];
+    T *dC = nullptr, *dA = nullptr, *dB = nullptr;
+    int rc = TC_OK;
+    if (hipMalloc(&dC, nC * sizeof(T)) != hipSuccess || hipMalloc(&dA, nA * sizeof(T)) != hipSuccess ||
+        hipMalloc(&dB, nB * sizeof(T)) != hipSuccess) {
+        rc = tc_fail(TC_ERR_ALLOC, "device allocation failed");
+    } else if (hipMemcpy(dC, hC, nC * sizeof(T), hipMemcpyHostToDevice) != hipSuccess ||
+               hipMemcpy(dA, hA, nA * sizeof(T), hipMemcpyHostToDevice) != hipSuccess ||
+               hipMemcpy(dB, hB, nB * sizeof(T), hipMemcpyHostToDevice) != hipSuccess) {
+        rc = tc_fail(TC_ERR_ALLOC, "host to device copy failed");
+    } else {
+        rc = tc_run<Cfg>(sizes, dC, dA, dB, 0, TC_VARIANT_AUTO);
+        if (rc == TC_OK && hipMemcpy(hC, dC, nC * sizeof(T), hipMemcpyDeviceToHost) != hipSuccess)
+            rc = tc_fail(TC_ERR_LAUNCH, "kernel execution or device to host copy failed");
+    }
+    if (dC) (void)hipFree(dC);
+    if (dA) (void)hipFree(dA);
+    if (dB) (void)hipFree(dB);
+    return rc;
+}
+
+}  // namespace cogent

@@ -1,0 +1,135 @@
+// HIP source emitter: one translation unit per contraction expression.
+//
+// Counterpart of cogent/src/codes/tc_gen_code.py:22-447, which writes
+// `temp__NN.cu` with #defines, four kernels, the host caller and the public
+// interface.  Here the per-expression text is a configuration struct (index
+// roles, tiles, wavefront layout, LDS layouts chosen by the mapping pass) that
+// instantiates the hand-written gfx950 kernel templates, plus the same public
+// entry point: `sd_t_d2_fusion_(int size_<idx>..., T* out, T* a, T* b, int, int)`
+// (cogent/src/codes/kernels/tc_interface.py:1444-1516) -- taking DEVICE pointers.
+#include "tc_ir.hpp"
+#include <sstream>
+
+namespace cogent {
+
+static std::string table(const char* name, const std::vector<int>& v)
+{
+    std::ostringstream o;
+    o << "    static constexpr __host__ __device__ int " << name << "(int i) { constexpr int v[" << (v.empty() ? 1 : v.size()) << "] = {";
+    if (v.empty()) o << "0";
+    for (size_t i = 0; i < v.size(); i++) o << (i ? ", " : "") << v[i];
+    o << "}; return v[i]; }\n";
+    return o.str();
+}
+
+static int pos_in(const std::vector<int>& v, int id)
+{
+    for (int i = 0; i < (int)v.size(); i++) if (v[i] == id) return i;
+    return -1;
+}
+
+static std::string c_escape(const std::string& s)
+{
+    std::string o;
+    for (char ch : s) {
+        if (ch == '"' || ch == '\\') { o.push_back('\\'); o.push_back(ch); }
+        else if (ch == '\n') o += "\\n";
+        else o.push_back(ch);
+    }
+    return o;
+}
+
+std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, const std::string& unique_name)
+{
+    std::ostringstream o;
+    const char* T = t == DType::F64 ? "double" : "float";
+    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
+    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
+
+    o << "// Emitted by cogent-mi355 for gfx950.  Do not edit: regenerate from the expression.\n";
+    o << "//   " << c.text << "\n";
+    o << "//   element type " << T << ", mapping " << m.spec() << "\n";
+    o << "#include \"tc_launch.hpp\"\n\n";
+    o << "namespace {\n";
+    o << "struct Cfg {\n";
+    o << "    typedef " << T << " T;\n";
+    o << "    static constexpr int NIDX = " << c.n_idx() << ", SIGN = " << c.sign << ";\n";
+    o << "    static constexpr bool X_IS_A = " << (m.x_is_a ? "true" : "false") << ";\n";
+    o << "    // tensors in memory order (index ids, fastest first)\n";
+    o << "    static constexpr int CR = " << c.out_idx.size() << ", AR = " << c.a_idx.size() << ", BR = " << c.b_idx.size() << ";\n";
+    o << table("c_id", c.out_idx) << table("a_id", c.a_idx) << table("b_id", c.b_idx) << table("sum_id", c.int_idx);
+    o << "    // composite tiles (fastest first): X side = externals of the input that holds C's fastest index\n";
+    o << "    static constexpr int NX = " << m.x_ids.size() << ", NY = " << m.y_ids.size() << ", NK = " << m.k_ids.size() << ";\n";
+    o << table("x_id", m.x_ids) << table("x_tile", m.x_tiles);
+    o << table("y_id", m.y_ids) << table("y_tile", m.y_tiles);
+    o << table("k_id", m.k_ids) << table("k_tile", m.k_tiles);
+    o << "    static constexpr int BX = " << m.BX << ", BY = " << m.BY << ", BK = " << m.BK << ";\n";
+    o << "    static constexpr int BXP = " << m.BXP << ", BYP = " << m.BYP << ", BKP = " << m.BKP << ";\n";
+
+    auto operand = [&](const char* p, const std::vector<int>& op, const std::vector<int>& e_ids, const std::vector<int>& e_tiles) {
+        std::vector<int> ids, tiles, isk, mul;
+        for (int id : op) {
+            ids.push_back(id);
+            int q;
+            if ((q = pos_in(m.k_ids, id)) >= 0) {
+                tiles.push_back(m.k_tiles[q]); isk.push_back(1);
+                int mm = 1; for (int j = 0; j < q; j++) mm *= m.k_tiles[j];
+                mul.push_back(mm);
+            } else {
+                q = pos_in(e_ids, id);
+                tiles.push_back(e_tiles[q]); isk.push_back(0);
+                int mm = 1; for (int j = 0; j < q; j++) mm *= e_tiles[j];
+                mul.push_back(mm);
+            }
+        }
+        o << "    static constexpr int " << p << "R = " << op.size() << ";\n";
+        std::string s(1, (char)tolower(p[0]));
+        o << table((s + "o_id").c_str(), ids) << table((s + "o_tile").c_str(), tiles)
+          << table((s + "o_isk").c_str(), isk) << table((s + "o_mul").c_str(), mul);
+    };
+    o << "    // the X- and Y-side operands in their own memory order: id, tile, contracted?, weight in the composite coordinate\n";
+    operand("X", xop, m.x_ids, m.x_tiles);
+    operand("Y", yop, m.y_ids, m.y_tiles);
+    o << "    static constexpr int WX = " << m.WX << ", WY = " << m.WY << ", TX = " << m.TX << ", TY = " << m.TY << ", NT = " << 64 * m.WX * m.WY << ";\n";
+    o << "    static constexpr int MI = " << m.MI << ";\n";
+    o << "    static constexpr int LAYX = " << m.layx << ", LDX = " << m.ldx << ", LAYY = " << m.layy << ", LDY = " << m.ldy << ";\n";
+    o << "};\n";
+    o << "}  // namespace\n\n";
+
+    // parameter lists
+    std::ostringstream params, sizes;
+    for (int i = 0; i < c.n_idx(); i++) {
+        params << "int size_" << c.indices[i].name << ", ";
+        sizes << (i ? ", " : "") << "size_" << c.indices[i].name;
+    }
+    params << T << "* " << c.out_name << ", " << T << "* " << c.a_name << ", " << T << "* " << c.b_name
+           << ", int cond_kernel_1, int opt_register_transpose";
+
+    o << "extern \"C\" {\n\n";
+    o << "// Public entry point, same name and argument order as the reference's generated interface;\n";
+    o << "// the three pointers are DEVICE pointers, the launch goes to the default stream and the call\n";
+    o << "// returns without synchronising.  Computes " << c.out_name << " " << c.op << " sum(" << c.a_name << " * " << c.b_name << ").  Returns 0 on success.\n";
+    o << "int sd_t_d2_fusion_(" << params.str() << ")\n{\n";
+    o << "    (void)cond_kernel_1; (void)opt_register_transpose;\n";
+    o << "    const int sizes[" << c.n_idx() << "] = {" << sizes.str() << "};\n";
+    o << "    return cogent::tc_run<Cfg>(sizes, " << c.out_name << ", " << c.a_name << ", " << c.b_name << ", 0, cogent::TC_VARIANT_AUTO);\n}\n\n";
+    o << "// Host-pointer form with the reference's behaviour: allocate, copy in (C included), run, copy C back, free.\n";
+    o << "int sd_t_d2_fusion_host_(" << params.str() << ")\n{\n";
+    o << "    (void)cond_kernel_1; (void)opt_register_transpose;\n";
+    o << "    const int sizes[" << c.n_idx() << "] = {" << sizes.str() << "};\n";
+    o << "    return cogent::tc_run_host<Cfg>(sizes, " << c.out_name << ", " << c.a_name << ", " << c.b_name << ");\n}\n\n";
+    o << "// Array form for drivers that load several expressions: sizes[] in entry-point order.\n";
+    o << "int cogent_run(const int* sizes, int n_sizes, void* C, const void* A, const void* B, void* stream, int variant)\n{\n";
+    o << "    if (!sizes || n_sizes != Cfg::NIDX) return cogent::tc_fail(cogent::TC_ERR_NULL_POINTER, \"sizes[] must hold one extent per index\");\n";
+    o << "    return cogent::tc_run<Cfg>(sizes, C, A, B, (hipStream_t)stream, variant);\n}\n\n";
+    o << "int cogent_" << unique_name << "_run(const int* sizes, int n_sizes, void* C, const void* A, const void* B, void* stream, int variant)\n{\n";
+    o << "    return cogent_run(sizes, n_sizes, C, A, B, stream, variant);\n}\n\n";
+    o << "int cogent_num_indices(void) { return Cfg::NIDX; }\n";
+    o << "const char* cogent_last_error(void) { return cogent::tc_error_buffer(); }\n";
+    o << "const char* cogent_expression(void) { return \"" << c_escape(c.text) << "\"; }\n";
+    o << "const char* cogent_info(void) { return \"" << c_escape(mapping_json(c, t, m)) << "\"; }\n";
+    o << "\n}  // extern \"C\"\n";
+    return o.str();
+}
+
+}  // namespace cogent

@@ -1,0 +1,99 @@
+// Intermediate representation shared by the parser, the mapping pass and the emitter.
+#pragma once
+#include <string>
+#include <vector>
+
+namespace cogent {
+
+// One index of a contraction.  Ids are dense: output indices in output order
+// first, then the contracted ("internal") indices in sum() order -- the order
+// in which the generated entry point takes its `int size_*` arguments
+// (cogent/src/codes/kernels/tc_interface.py:1459-1492).
+struct Index {
+    std::string name;
+    int rep_size = 0;        // representative problem size from the expression (mapping only)
+    bool internal = false;   // summed over
+};
+
+// `out [..] op sum(..) * a [..] * b [..];`, the record of
+// cogent/src/algs/bases/tc_gen_inputs.py:108.  Index lists hold ids, FASTEST
+// index first (the reference's tensors are column-major).
+struct Contraction {
+    std::string text;
+    std::string out_name, a_name, b_name;
+    std::string op;          // "+=" or "-="
+    int sign = 1;
+    std::vector<Index> indices;
+    std::vector<int> out_idx, int_idx, a_idx, b_idx;
+
+    int n_idx() const { return (int)indices.size(); }
+    bool in_a(int id) const { for (int v : a_idx) if (v == id) return true; return false; }
+    bool in_b(int id) const { for (int v : b_idx) if (v == id) return true; return false; }
+};
+
+enum class DType { F64, F32 };
+
+// gfx950 (MI355X) figures the mapping pass sizes tiles against.
+struct ArchGfx950 {
+    int wave = 64;
+    int n_cu = 256;
+    int simd_per_cu = 4;
+    int lds_bytes_per_cu = 160 * 1024;
+    int lds_bytes_per_block = 64 * 1024;     // static __shared__ limit
+    int max_threads_per_block = 1024;
+    int max_waves_per_cu = 32;
+    int vgpr_per_lane = 512;                 // unified VGPR+AGPR file at one wave per SIMD
+    double clock_hz = 2.4e9;
+    double hbm_bytes_per_s = 8.0e12;         // published peak
+    double hbm_sustained_fraction = 0.70;    // what a plain copy kernel reaches on the part
+    double l2_bytes_per_s = 14.0e12;         // aggregate L2/Infinity-Cache rate for re-read operand slices
+    double lds_bytes_per_clk_cu = 128.0;
+    double mfma_f64_flops = 78.6e12;
+    double mfma_f32_flops = 157.3e12;
+};
+
+// One index-to-tile mapping for gfx950: the counterpart of the reference's
+// Config record (cogent/src/algs/bases/class_configuration.py:4-65), with
+// wave / MFMA tiling and LDS layouts in place of TB_X/TB_Y/REG_X/REG_Y.
+struct Mapping {
+    bool x_is_a = true;                       // X side = the input that holds the output's fastest index
+    std::vector<int> x_ids, x_tiles;          // composite order, fastest first
+    std::vector<int> y_ids, y_tiles;
+    std::vector<int> k_ids, k_tiles;
+    int BX = 0, BY = 0, BK = 0;               // tile products
+    int BXP = 0, BYP = 0, BKP = 0;            // padded to MFMA granularity
+    int WX = 1, WY = 1, TX = 1, TY = 1;       // wavefront grid and MFMA tiles per wavefront
+    int MI = 0;                               // 0 f64 16x16x4, 1 f32 16x16x4, 2 f32 32x32x2
+    int layx = 0, ldx = 0, layy = 0, ldy = 0; // LDS layout per operand
+    // model outputs
+    double t_hbm = 0, t_l2 = 0, t_mfma = 0, t_lds = 0, tail_eff = 1, cost = 0;
+    long long n_blocks = 0; int lds_bytes = 0; int blocks_per_cu = 0;
+    int steps_main_loop = 0;
+    std::string spec() const;                 // compact text form, parseable by mapping_from_spec
+};
+
+// ---- parser (tc_parse.cpp)
+// Reads an expression file the way the reference does: lines starting with '#'
+// are skipped, every other line is one expression.  Returns false and sets err
+// on the inputs the reference cannot process.
+bool parse_expression_line(const std::string& line, Contraction& out, std::string& err);
+bool parse_expression_file(const std::string& path, std::vector<Contraction>& out, std::string& err);
+bool parse_expression_text(const std::string& text, std::vector<Contraction>& out, std::string& err);
+
+// ---- mapping (tc_mapping.cpp)
+std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const ArchGfx950& arch);
+void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& m);
+// rank < 0: cheapest by the model; otherwise the rank-th of the sorted list
+bool select_mapping(const Contraction& c, DType t, const ArchGfx950& arch, int rank, Mapping& out, std::string& err);
+bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, const std::string& spec, Mapping& out, std::string& err);
+bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const Mapping& m, std::string& err);
+std::string mapping_json(const Contraction& c, DType t, const Mapping& m);
+
+// ---- emitter (tc_emit.cpp)
+std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, const std::string& unique_name);
+
+// ---- accounting
+long long contraction_flops(const Contraction& c, const int* sizes);                 // 2 * prod(all extents)
+long long contraction_bytes(const Contraction& c, DType t, const int* sizes);        // sizeof(T) * (|A| + |B| + 2|C|)
+
+}  // namespace cogent

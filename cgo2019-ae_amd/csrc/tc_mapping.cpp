@@ -1,0 +1,487 @@
+// Index-to-tile mapping pass for gfx950.
+//
+// Plays the part of the reference's enumeration + pruning
+// (cogent/src/algs/bases/enumeration.py:15-278), cost model
+// (cogent/src/algs/bases/cost_models.py:11-631) and selection
+// (cogent/src/generators/configurations.py:254-289), re-derived for CDNA4:
+//
+//   reference (warp-32, 48 KB smem)            here (wave-64, MFMA, 160 KB LDS)
+//   ---------------------------------------    ----------------------------------------
+//   TB_X / TB_Y thread-block index lists       X / Y composite tiles, X = side of C's
+//   ("left" = input with the output FVI,         fastest index (same rule, enumeration.py:72-99)
+//    enumeration.py:72-99)
+//   REG_X / REG_Y per-thread register tile     TX x TY MFMA accumulator tiles per wavefront
+//   tile menus TB {4,8,16}, REG {1,2,4,6,8}    any divisor / power of two per index, tile
+//                                                products up to 512, padded to 16 or 32
+//   greedy prefix over consecutive indices     the same greedy prefix (full extents, then
+//   (enumeration.py:352-374)                     one partial index, then 1s), tried in C
+//                                                order and in operand order
+//   cost = DRAM transactions x thread blocks   time = max(HBM, L2 re-reads, MFMA, LDS) with
+//                                                coalescing, tail and latency-hiding terms
+//   limits: 64..1024 threads, 6144 elements    64..1024 threads, 64 KB LDS per block,
+//   of smem (tc_gen.py:167-196)                  accumulators within the VGPR file
+//
+// A single external index of an input may be given a tile smaller than its
+// extent, so the reference's x -> x1,x2 split (configurations.py:93-230) is not
+// needed: the grid takes the quotient.  The entry point keeps the un-split arity.
+#include "tc_ir.hpp"
+#include <algorithm>
+#include <array>
+#include <cmath>
+#include <cstdio>
+#include <map>
+#include <set>
+#include <sstream>
+
+namespace cogent {
+
+static int esize(DType t) { return t == DType::F64 ? 8 : 4; }
+static int ceil_div(int a, int b) { return (a + b - 1) / b; }
+static int round_up(int a, int b) { return ceil_div(a, b) * b; }
+
+struct MiInfo { int MT, KSTEP, NREG; double cycles; };
+static MiInfo mi_info(int mi)
+{
+    // cycles per instruction per SIMD implied by the published matrix peaks
+    // (78.6 TFLOP/s fp64, 157.3 TFLOP/s fp32 over 256 CUs x 4 SIMDs at 2.4 GHz)
+    if (mi == 0) return {16, 4, 4, 64.0};
+    if (mi == 1) return {16, 4, 4, 32.0};
+    return {32, 2, 16, 64.0};
+}
+
+std::string Mapping::spec() const
+{
+    std::ostringstream o;
+    auto side = [&](const char* tag, const std::vector<int>& ids, const std::vector<int>& tiles) {
+        o << tag << "=";
+        for (size_t i = 0; i < ids.size(); i++) o << (i ? "," : "") << ids[i] << ":" << tiles[i];
+        o << ";";
+    };
+    side("x", x_ids, x_tiles);
+    side("y", y_ids, y_tiles);
+    side("k", k_ids, k_tiles);
+    o << "w=" << WX << "x" << WY << ";t=" << TX << "x" << TY << ";mi=" << MI
+      << ";lx=" << layx << ";ly=" << layy;
+    return o.str();
+}
+
+static std::vector<int> tile_options(int ext, int cap)
+{
+    std::set<int> s;
+    for (int t = 1; t <= ext && t <= cap; t++) if (ext % t == 0) s.insert(t);
+    for (int t = 1; t < ext && t <= cap; t *= 2) s.insert(t);
+    if (ext <= cap) s.insert(ext);
+    return std::vector<int>(s.begin(), s.end());
+}
+
+struct SideCand { std::vector<int> ids, tiles; int B; };
+
+// greedy prefix: leading indices take their full extent, one index a partial tile, the rest 1
+static void prefix_candidates(const Contraction& c, const std::vector<int>& order, int maxB,
+                              std::vector<SideCand>& out)
+{
+    std::set<std::vector<int>> seen;
+    const int n = (int)order.size();
+    long long P = 1;
+    for (int p = 0; p < n; p++) {
+        const int ext = c.indices[order[p]].rep_size;
+        for (int t : tile_options(ext, maxB)) {
+            if (P * t > maxB) break;
+            SideCand sc;
+            sc.ids = order;
+            sc.tiles.assign(n, 1);
+            for (int j = 0; j < p; j++) sc.tiles[j] = c.indices[order[j]].rep_size;
+            sc.tiles[p] = t;
+            sc.B = (int)(P * t);
+            std::vector<int> key = sc.ids;
+            key.insert(key.end(), sc.tiles.begin(), sc.tiles.end());
+            if (seen.insert(key).second) out.push_back(sc);
+        }
+        P *= ext;
+        if (P > maxB) break;
+    }
+}
+
+static int pos_in(const std::vector<int>& v, int id)
+{
+    for (int i = 0; i < (int)v.size(); i++) if (v[i] == id) return i;
+    return -1;
+}
+
+// LDS leading dimension (elements) that keeps the MFMA operand reads free of bank conflicts.
+//   k-major (addr = k*LD + e): the rows read together by one half-wave must land in
+//   different bank groups: LD = 16 mod 32 for 8-byte elements; 16 mod 64 (16-wide tiles)
+//   or 32 mod 64 (32-wide tiles) for 4-byte elements.
+//   e-major (addr = e*LD + k): LD = BKP + 2 (8-byte, or 32-wide 4-byte tiles) or
+//   BKP + 4 (16-wide 4-byte tiles), bumped until LD/2 (resp. LD/4) is odd.
+static int lds_ld(int lay, int bep, int bkp, DType t, int mi)
+{
+    if (lay == 0) {
+        int mod = (t == DType::F64) ? 32 : 64;
+        int want = (t == DType::F64) ? 16 : (mi == 2 ? 32 : 16);
+        int ld = bep;
+        while (ld % mod != want) ld++;
+        return ld;
+    }
+    if (t == DType::F64 || mi == 2) {
+        int ld = bkp + 2;
+        while ((ld % 2) || ((ld / 2) % 2 == 0)) ld++;
+        return ld;
+    }
+    int ld = bkp + 4;
+    while ((ld % 4) || ((ld / 4) % 2 == 0)) ld++;
+    return ld;
+}
+
+static int fvi(const std::vector<int>& idx) { return idx.empty() ? -1 : idx[0]; }
+
+static void finish_geometry(const Contraction& c, DType t, Mapping& m)
+{
+    const MiInfo mi = mi_info(m.MI);
+    m.BX = 1; for (int v : m.x_tiles) m.BX *= v;
+    m.BY = 1; for (int v : m.y_tiles) m.BY *= v;
+    m.BK = 1; for (int v : m.k_tiles) m.BK *= v;
+    m.BXP = m.WX * m.TX * mi.MT;
+    m.BYP = m.WY * m.TY * mi.MT;
+    m.BKP = round_up(m.BK, mi.KSTEP);
+    m.ldx = lds_ld(m.layx, m.BXP, m.BKP, t, m.MI);
+    m.ldy = lds_ld(m.layy, m.BYP, m.BKP, t, m.MI);
+    const int ex = m.layx == 0 ? m.BKP * m.ldx : m.BXP * m.ldx;
+    const int ey = m.layy == 0 ? m.BKP * m.ldy : m.BYP * m.ldy;
+    m.lds_bytes = (ex + ey) * esize(t);
+    (void)c;
+}
+
+bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const Mapping& m, std::string& err)
+{
+    const MiInfo mi = mi_info(m.MI);
+    if ((t == DType::F64) != (m.MI == 0)) { err = "matrix instruction does not match the element type"; return false; }
+    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
+    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
+    std::vector<int> seen(c.n_idx(), 0);
+    auto side = [&](const std::vector<int>& ids, const std::vector<int>& tiles, const std::vector<int>& op, bool internal, const char* what) -> bool {
+        if (ids.size() != tiles.size()) { err = std::string(what) + ": ids and tiles differ in length"; return false; }
+        for (size_t i = 0; i < ids.size(); i++) {
+            int id = ids[i];
+            if (id < 0 || id >= c.n_idx()) { err = std::string(what) + ": unknown index id"; return false; }
+            if (c.indices[id].internal != internal) { err = std::string(what) + ": index '" + c.indices[id].name + "' is on the wrong side"; return false; }
+            if (pos_in(op, id) < 0) { err = std::string(what) + ": index '" + c.indices[id].name + "' is not in that operand"; return false; }
+            if (tiles[i] < 1) { err = std::string(what) + ": tile must be positive"; return false; }
+            seen[id]++;
+        }
+        return true;
+    };
+    if (!side(m.x_ids, m.x_tiles, xop, false, "x") || !side(m.y_ids, m.y_tiles, yop, false, "y")) return false;
+    if (!side(m.k_ids, m.k_tiles, xop, true, "k")) return false;
+    for (int i = 0; i < c.n_idx(); i++)
+        if (seen[i] != 1) { err = "index '" + c.indices[i].name + "' must be mapped exactly once"; return false; }
+    if (m.x_ids.empty()) { err = "the input holding the output's fastest index needs an external index"; return false; }
+    const int threads = 64 * m.WX * m.WY;
+    if (threads < 64 || threads > arch.max_threads_per_block) { err = "threads per block outside 64..1024"; return false; }
+    if (m.BXP < m.BX || m.BYP < m.BY) { err = "wavefront tiling does not cover the block tile"; return false; }
+    if (m.lds_bytes > arch.lds_bytes_per_block) { err = "LDS slices exceed 64 KB per block"; return false; }
+    const int acc_regs = m.TX * m.TY * mi.NREG * (esize(t) / 4);
+    // 512 registers per lane and SIMD are shared by the block's wavefronts on that SIMD;
+    // the accumulators may take half of a wavefront's share
+    const int waves_per_simd = ceil_div(m.WX * m.WY, arch.simd_per_cu);
+    const int reg_budget = std::min(512, arch.vgpr_per_lane / waves_per_simd);
+    if (acc_regs > 256 || acc_regs * 2 > reg_budget) { err = "accumulator tiles exceed the register budget per lane"; return false; }
+    if (m.layx < 0 || m.layx > 1 || m.layy < 0 || m.layy > 1) { err = "unknown LDS layout"; return false; }
+    return true;
+}
+
+void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& m)
+{
+    const MiInfo mi = mi_info(m.MI);
+    const double s = esize(t);
+    auto ext = [&](int id) { return (double)c.indices[id].rep_size; };
+    auto tile_of = [&](int id) -> int {
+        int p;
+        if ((p = pos_in(m.x_ids, id)) >= 0) return m.x_tiles[p];
+        if ((p = pos_in(m.y_ids, id)) >= 0) return m.y_tiles[p];
+        if ((p = pos_in(m.k_ids, id)) >= 0) return m.k_tiles[p];
+        return 1;
+    };
+    double nC = 1, nA = 1, nB = 1;
+    for (int id : c.out_idx) nC *= ext(id);
+    for (int id : c.a_idx) nA *= ext(id);
+    for (int id : c.b_idx) nB *= ext(id);
+
+    long long nblocks = 1;
+    for (size_t i = 0; i < m.x_ids.size(); i++) nblocks *= ceil_div(c.indices[m.x_ids[i]].rep_size, m.x_tiles[i]);
+    for (size_t i = 0; i < m.y_ids.size(); i++) nblocks *= ceil_div(c.indices[m.y_ids[i]].rep_size, m.y_tiles[i]);
+    long long nkb = 1;
+    for (size_t i = 0; i < m.k_ids.size(); i++) nkb *= ceil_div(c.indices[m.k_ids[i]].rep_size, m.k_tiles[i]);
+    m.n_blocks = nblocks;
+    m.steps_main_loop = (int)nkb;
+
+    // contiguous run of C covered by neighbouring lanes (elements)
+    double run = 1;
+    if (!m.x_ids.empty() && m.x_ids[0] == c.out_idx[0]) {
+        run = m.x_tiles[0];
+        size_t j = 0;
+        while (j + 1 < m.x_ids.size() && m.x_tiles[j] == c.indices[m.x_ids[j]].rep_size &&
+               pos_in(c.out_idx, m.x_ids[j + 1]) == pos_in(c.out_idx, m.x_ids[j]) + 1) {
+            run *= m.x_tiles[j + 1];
+            j++;
+        }
+    }
+    const double seg_bytes = std::min(run, (double)mi.MT) * s;
+    const double c_l1_eff = std::min(1.0, seg_bytes / 128.0);
+    // contiguous chunk of C owned by one block (bytes): whole 128-byte lines or not
+    double chunk = 1;
+    for (int id : c.out_idx) {
+        const int tl = tile_of(id);
+        chunk *= tl;
+        if (tl != c.indices[id].rep_size) break;
+    }
+    const double c_hbm_eff = std::min(1.0, chunk * s / 128.0);
+
+    // resident blocks per CU
+    const int W = m.WX * m.WY;
+    const int acc_regs = m.TX * m.TY * mi.NREG * (int)(s / 4);
+    const int slots = (int)std::ceil((double)m.BK * (m.BX + m.BY) / (64.0 * W));
+    const int regs = acc_regs + slots * (int)(s / 4) * 2 + (m.TX + m.TY) * (int)(s / 4) + 48;
+    int waves_per_simd = std::max(1, std::min(8, arch.vgpr_per_lane / std::max(regs, 64)));
+    int r = std::min(arch.lds_bytes_per_cu / std::max(m.lds_bytes, 1), arch.max_waves_per_cu / W);
+    r = std::min(r, std::max(1, waves_per_simd * arch.simd_per_cu / W));
+    r = std::max(r, 1);
+    m.blocks_per_cu = r;
+
+    const double bw = arch.hbm_bytes_per_s * arch.hbm_sustained_fraction;
+    // bytes in flight needed to cover HBM latency: about 48 KB per CU
+    const double inflight = (double)r * m.BX * m.BY * s + (double)r * m.BK * (m.BX + m.BY) * s;
+    const double lat_scale = std::min(1.0, inflight / (48.0 * 1024.0));
+    m.t_hbm = ((nA + nB) * s + 2.0 * nC * s / c_hbm_eff) / (bw * lat_scale);
+    const double l1_bw = 64.0 * arch.n_cu * arch.clock_hz;
+    const double t_l1 = 2.0 * nC * s / (l1_bw * c_l1_eff);
+
+    // operand slices are re-read by every block that needs them; they mostly hit in L2 / Infinity Cache
+    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
+    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
+    auto op_eff = [&](const std::vector<int>& op) {
+        double rn = tile_of(op[0]);
+        size_t j = 0;
+        while (j + 1 < op.size() && tile_of(op[j]) == c.indices[op[j]].rep_size) { rn *= tile_of(op[j + 1]); j++; }
+        return std::min(1.0, rn * s / 128.0);
+    };
+    const double stage_x = (double)nblocks * nkb * m.BK * m.BX * s;
+    const double stage_y = (double)nblocks * nkb * m.BK * m.BY * s;
+    m.t_l2 = stage_x / (arch.l2_bytes_per_s * op_eff(xop)) + stage_y / (arch.l2_bytes_per_s * op_eff(yop));
+
+    const double simd_busy = std::min(1.0, (double)(W * r) / (arch.simd_per_cu * std::ceil((double)(W * r) / arch.simd_per_cu)));
+    const double n_mfma = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * (m.BXP / mi.MT) * (m.BYP / mi.MT);
+    m.t_mfma = n_mfma * mi.cycles / (arch.n_cu * arch.simd_per_cu * arch.clock_hz) / simd_busy;
+
+    const double lds_reads = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * W * (m.TX + m.TY) * 64.0 * s;
+    m.t_lds = (lds_reads + stage_x + stage_y) / (arch.lds_bytes_per_clk_cu * arch.n_cu * arch.clock_hz);
+
+    const double slots_total = (double)arch.n_cu * r;
+    const double rounds = std::ceil((double)nblocks / slots_total);
+    m.tail_eff = (double)nblocks / (rounds * slots_total);
+
+    const double parts[4] = {m.t_hbm + 0.0, m.t_l2, m.t_mfma, m.t_lds};
+    double mx = std::max(t_l1, 0.0), sum = t_l1;
+    for (double p : parts) { mx = std::max(mx, p); sum += p; }
+    // the slowest pipe sets the pace; the others overlap imperfectly
+    m.cost = (mx + 0.15 * (sum - mx)) / std::max(m.tail_eff, 0.05) + 2.0e-6;
+}
+
+static void wave_layouts(int nx, int ny, int max_acc_tiles, std::vector<std::array<int, 4>>& out)
+{
+    for (int wx = 1; wx <= nx && wx <= 16; wx++) {
+        if (nx % wx) continue;
+        for (int wy = 1; wy <= ny && wx * wy <= 16; wy++) {
+            if (ny % wy) continue;
+            const int tx = nx / wx, ty = ny / wy;
+            if (tx * ty > max_acc_tiles) continue;
+            out.push_back({wx, wy, tx, ty});
+        }
+    }
+}
+
+std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const ArchGfx950& arch)
+{
+    std::vector<Mapping> out;
+    if (c.out_idx.empty()) return out;
+    const bool x_is_a = c.in_a(c.out_idx[0]);
+    const std::vector<int>& xop = x_is_a ? c.a_idx : c.b_idx;
+    const std::vector<int>& yop = x_is_a ? c.b_idx : c.a_idx;
+
+    auto externals_in = [&](const std::vector<int>& op, bool by_c_order) {
+        std::vector<int> v;
+        if (by_c_order) { for (int id : c.out_idx) if (pos_in(op, id) >= 0) v.push_back(id); }
+        else            { for (int id : op) if (!c.indices[id].internal) v.push_back(id); }
+        return v;
+    };
+    std::vector<std::vector<int>> x_orders, y_orders, k_orders;
+    x_orders.push_back(externals_in(xop, true));          // X must start at C's fastest index
+    for (int by_c = 1; by_c >= 0; by_c--) {
+        std::vector<int> o = externals_in(yop, by_c != 0);
+        if (std::find(y_orders.begin(), y_orders.end(), o) == y_orders.end()) y_orders.push_back(o);
+    }
+    // K composite order: an index that is the fastest one of an operand goes first
+    {
+        std::vector<int> base = c.int_idx, o1, o2;
+        auto order_with_first = [&](int first) {
+            std::vector<int> o;
+            if (first >= 0 && c.indices[first].internal) o.push_back(first);
+            for (int id : xop) if (c.indices[id].internal && pos_in(o, id) < 0) o.push_back(id);
+            return o;
+        };
+        std::vector<std::vector<int>> cand = {order_with_first(fvi(xop)), order_with_first(fvi(yop)), base};
+        std::vector<int> by_y;
+        for (int id : yop) if (c.indices[id].internal) by_y.push_back(id);
+        cand.push_back(by_y);
+        for (auto& o : cand)
+            if (o.size() == c.int_idx.size() && std::find(k_orders.begin(), k_orders.end(), o) == k_orders.end()) k_orders.push_back(o);
+    }
+
+    std::vector<SideCand> xc, yc, kc;
+    for (auto& o : x_orders) prefix_candidates(c, o, 512, xc);
+    for (auto& o : y_orders) prefix_candidates(c, o, 512, yc);
+    for (auto& o : k_orders) prefix_candidates(c, o, 64, kc);
+    // an input without external indices (matrix-vector shapes) or without a summed index: one empty tile
+    if (yc.empty()) yc.push_back(SideCand{{}, {}, 1});
+    if (kc.empty()) kc.push_back(SideCand{{}, {}, 1});
+    int max_bx = 1, max_by = 1, max_bk = 1;
+    for (auto& s : xc) max_bx = std::max(max_bx, s.B);
+    for (auto& s : yc) max_by = std::max(max_by, s.B);
+    for (auto& s : kc) max_bk = std::max(max_bk, s.B);
+
+    const std::vector<int> mis = (t == DType::F64) ? std::vector<int>{0} : std::vector<int>{1, 2};
+    for (int miv : mis) {
+        const MiInfo mi = mi_info(miv);
+        const int max_acc_tiles = 128 / (mi.NREG * (esize(t) / 4));     // 128 accumulator registers per lane
+        for (const SideCand& kx : kc) {
+            if (kx.B < std::min(4, max_bk)) continue;
+            for (const SideCand& sx : xc) {
+                if (sx.B < std::min(8, max_bx)) continue;
+                const int nx = ceil_div(sx.B, mi.MT);
+                if ((double)sx.B / (nx * mi.MT) < 0.7 && sx.B != max_bx) continue;
+                for (const SideCand& sy : yc) {
+                    if (sy.B < std::min(8, max_by)) continue;
+                    const int ny = ceil_div(sy.B, mi.MT);
+                    if ((double)sy.B / (ny * mi.MT) < 0.7 && sy.B != max_by) continue;
+                    std::vector<std::array<int, 4>> wl;
+                    wave_layouts(nx, ny, max_acc_tiles, wl);
+                    for (auto& w : wl) {
+                        Mapping m;
+                        m.x_is_a = x_is_a;
+                        m.x_ids = sx.ids; m.x_tiles = sx.tiles;
+                        m.y_ids = sy.ids; m.y_tiles = sy.tiles;
+                        m.k_ids = kx.ids; m.k_tiles = kx.tiles;
+                        m.WX = w[0]; m.WY = w[1]; m.TX = w[2]; m.TY = w[3];
+                        m.MI = miv;
+                        // k-fast LDS layout when the operand's fastest index is the leading K index with a real tile
+                        m.layx = (!kx.ids.empty() && kx.ids[0] == fvi(xop) && kx.tiles[0] >= 4) ? 1 : 0;
+                        m.layy = (!kx.ids.empty() && kx.ids[0] == fvi(yop) && kx.tiles[0] >= 4) ? 1 : 0;
+                        finish_geometry(c, t, m);
+                        std::string err;
+                        if (!check_mapping(c, t, arch, m, err)) continue;
+                        cost_model(c, t, arch, m);
+                        out.push_back(m);
+                    }
+                }
+            }
+        }
+    }
+    // cheapest first; ties go to fewer main-loop steps (configurations.py:260-283)
+    std::stable_sort(out.begin(), out.end(), [](const Mapping& a, const Mapping& b) {
+        if (a.cost != b.cost) return a.cost < b.cost;
+        return a.steps_main_loop < b.steps_main_loop;
+    });
+    return out;
+}
+
+bool select_mapping(const Contraction& c, DType t, const ArchGfx950& arch, int rank, Mapping& out, std::string& err)
+{
+    std::vector<Mapping> all = enumerate_mappings(c, t, arch);
+    if (all.empty()) { err = "no admissible mapping for this expression"; return false; }
+    if (rank >= 0 && rank < (int)all.size()) out = all[rank];   // manual pick, configurations.py:285-289
+    else out = all[0];
+    return true;
+}
+
+// spec grammar: x=<id>:<tile>,...;y=...;k=...;w=<WX>x<WY>;t=<TX>x<TY>;mi=<n>;lx=<0|1>;ly=<0|1>
+// index ids may also be given by name.
+bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, const std::string& spec, Mapping& m, std::string& err)
+{
+    m = Mapping();
+    m.x_is_a = c.in_a(c.out_idx[0]);
+    m.MI = (t == DType::F64) ? 0 : 1;
+    int lx = -1, ly = -1;
+    std::istringstream is(spec);
+    std::string field;
+    auto index_of = [&](const std::string& s) -> int {
+        for (int i = 0; i < c.n_idx(); i++) if (c.indices[i].name == s) return i;
+        bool digits = !s.empty();
+        for (char ch : s) if (ch < '0' || ch > '9') digits = false;
+        if (digits) { int v = atoi(s.c_str()); if (v < c.n_idx()) return v; }
+        return -1;
+    };
+    while (std::getline(is, field, ';')) {
+        if (field.empty()) continue;
+        size_t eq = field.find('=');
+        if (eq == std::string::npos) { err = "mapping spec field without '=': " + field; return false; }
+        std::string key = field.substr(0, eq), val = field.substr(eq + 1);
+        if (key == "x" || key == "y" || key == "k") {
+            std::vector<int>& ids = key == "x" ? m.x_ids : key == "y" ? m.y_ids : m.k_ids;
+            std::vector<int>& tiles = key == "x" ? m.x_tiles : key == "y" ? m.y_tiles : m.k_tiles;
+            std::istringstream vs(val);
+            std::string item;
+            while (std::getline(vs, item, ',')) {
+                size_t colon = item.find(':');
+                if (colon == std::string::npos) { err = "mapping spec item without ':': " + item; return false; }
+                int id = index_of(item.substr(0, colon));
+                if (id < 0) { err = "mapping spec names an unknown index: " + item; return false; }
+                ids.push_back(id);
+                tiles.push_back(atoi(item.substr(colon + 1).c_str()));
+            }
+        } else if (key == "w" || key == "t") {
+            int a = 0, b = 0;
+            if (sscanf(val.c_str(), "%dx%d", &a, &b) != 2 || a < 1 || b < 1) { err = "mapping spec: bad " + key; return false; }
+            if (key == "w") { m.WX = a; m.WY = b; } else { m.TX = a; m.TY = b; }
+        } else if (key == "mi") m.MI = atoi(val.c_str());
+        else if (key == "lx") lx = atoi(val.c_str());
+        else if (key == "ly") ly = atoi(val.c_str());
+        else { err = "mapping spec: unknown key " + key; return false; }
+    }
+    if (m.MI < 0 || m.MI > 2) { err = "mapping spec: unknown matrix instruction"; return false; }
+    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
+    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
+    if (m.x_ids.empty()) { err = "mapping spec must give x"; return false; }
+    m.layx = lx >= 0 ? lx : ((!m.k_ids.empty() && m.k_ids[0] == fvi(xop) && m.k_tiles[0] >= 4) ? 1 : 0);
+    m.layy = ly >= 0 ? ly : ((!m.k_ids.empty() && m.k_ids[0] == fvi(yop) && m.k_tiles[0] >= 4) ? 1 : 0);
+    finish_geometry(c, t, m);
+    if (!check_mapping(c, t, arch, m, err)) return false;
+    cost_model(c, t, arch, m);
+    return true;
+}
+
+std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
+{
+    std::ostringstream o;
+    auto side = [&](const char* tag, const std::vector<int>& ids, const std::vector<int>& tiles) {
+        o << "\"" << tag << "\": [";
+        for (size_t i = 0; i < ids.size(); i++)
+            o << (i ? ", " : "") << "[\"" << c.indices[ids[i]].name << "\", " << tiles[i] << "]";
+        o << "]";
+    };
+    o << "{\"dtype\": \"" << (t == DType::F64 ? "f64" : "f32") << "\", \"x_operand\": \"" << (m.x_is_a ? c.a_name : c.b_name) << "\", ";
+    side("x", m.x_ids, m.x_tiles); o << ", ";
+    side("y", m.y_ids, m.y_tiles); o << ", ";
+    side("k", m.k_ids, m.k_tiles); o << ", ";
+    const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
+    o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
+      << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
+      << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
+      << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6
+      << ", \"t_lds_us\": " << m.t_lds * 1e6 << ", \"tail_eff\": " << m.tail_eff << ", \"cost_us\": " << m.cost * 1e6 << "}, "
+      << "\"spec\": \"" << m.spec() << "\"}";
+    return o.str();
+}
+
+}  // namespace cogent
