@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Benchmark driver: GFLOP/s of one tensor contraction on one MI355X, with its roofline fraction.
+
+A "step" is one launch of the contraction through the per-expression C-ABI object, inputs resident
+in HBM.  The headline workload is BASELINE config 2 (fp64, 4-D output, one contracted index, all
+extents 72); the other BASELINE configs are timed the same way and listed under "all_configs".
+
+  value          flops / wall-clock time of K back-to-back launches (flops = 2 * product of extents,
+                 cogent/src/codes/kernels/tc_interface.py:289-305; cogent/data-tccg.py:49)
+  roofline       algorithmic bytes sizeof(T) * (|A| + |B| + 2|C|) per launch / mean per-launch
+                 duration from HIP events recorded between launches on the launch stream
+  cpu_baseline   the reference's host nested-loop contraction (CPU oracle) timed on this box's cores
+                 on the same seeded inputs, and used to verify the GPU result element by element
+
+Output buffers are rotated through a pool larger than the 256 MB Infinity Cache so that no launch
+finds its output tensor cached by the previous one.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "cgo2019-ae_amd"))
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3}
+TOL = {"f64": 1e-12, "f32": 1e-5}
+HEADLINE = "cfg2_f64"
+
+
+def read_traffic(name):
+    """HBM bytes per launch from the rocprofv3 counter summary under profiles/, or None."""
+    path = os.path.join(ROOT, "profiles", "traffic_%s.txt" % name)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("hbm_bytes_per_launch:"):
+            return float(line.split(":")[1])
+    return None
+
+
+class Workload:
+    def __init__(self, pkg, tools, entry, sizes):
+        import numpy as np
+        import torch
+        self.name = entry["name"]
+        self.sizes = list(sizes)
+        self.ex = pkg.Expression(self.name)
+        self.plan = tools.plan(pkg.expression_text(self.name), entry["dtype"])
+        self.dtype = self.ex.dtype
+        np_dtype = np.float64 if self.dtype == "f64" else np.float32
+        names = self.plan.info["out_idx"] + self.plan.info["sum_idx"]
+        ext = dict(zip(names, self.sizes))
+        count = lambda idx: int(np.prod([ext[i] for i in idx], dtype=np.int64))
+        self.nC, self.nA, self.nB = count(self.plan.info["out_idx"]), count(self.plan.info["a_idx"]), count(self.plan.info["b_idx"])
+        self.flops = self.plan.flops(self.sizes)
+        self.bytes = self.plan.bytes(self.sizes)
+        esize = 8 if self.dtype == "f64" else 4
+        # seeds 1, 2, 3 for A, B, C; C starts at zero unless the config says it is seeded
+        self.hA = tools.fill_uniform(np.empty(self.nA, np_dtype), 1)
+        self.hB = tools.fill_uniform(np.empty(self.nB, np_dtype), 2)
+        if entry.get("c_init") == "seeded":
+            self.hC = tools.fill_uniform(np.empty(self.nC, np_dtype), 3)
+        else:
+            self.hC = np.zeros(self.nC, np_dtype)
+        self.dA = torch.from_numpy(self.hA).cuda()
+        self.dB = torch.from_numpy(self.hB).cuda()
+        n_rot = max(2, min(8, int(1.2e9 // (self.nC * esize)) + 1))
+        c0 = torch.from_numpy(self.hC).cuda()
+        self.dC = [c0] + [c0.clone() for _ in range(n_rot - 1)]
+
+    def c_ptrs(self):
+        return [c.data_ptr() for c in self.dC]
+
+    def launch(self, i):
+        rc = self.ex.run(self.sizes, self.dC[i % len(self.dC)].data_ptr(), self.dA.data_ptr(), self.dB.data_ptr(), None, 0)
+        if rc:
+            raise RuntimeError("launch failed (%d): %s" % (rc, self.ex.last_error()))
+
+    def reset_c(self):
+        import torch
+        src = torch.from_numpy(self.hC).cuda()
+        for c in self.dC:
+            c.copy_(src)
+        torch.cuda.synchronize()
+
+
+def roofline(w, mean_ms):
+    sec = mean_ms * 1e-3
+    gbs = w.bytes / sec / 1e9
+    tfl = w.flops / sec / 1e12
+    hbm = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    mfma = {"bound": "mfma", "achieved": round(tfl, 3), "peak": MFMA_PEAK_TFLOPS[w.dtype], "unit": "TFLOP/s",
+            "frac": round(tfl / MFMA_PEAK_TFLOPS[w.dtype], 4)}
+    t_hbm = w.bytes / (HBM_PEAK_GBS * 1e9)
+    t_mfma = w.flops / (MFMA_PEAK_TFLOPS[w.dtype] * 1e12)
+    return (hbm, mfma) if t_hbm >= t_mfma else (mfma, hbm)
+
+
+def time_workload(driver, w, warmup, iters):
+    st = driver.time(w.ex, w.sizes, w.c_ptrs(), w.dA.data_ptr(), w.dB.data_ptr(), warmup, iters)
+    primary, secondary = roofline(w, st["mean_ms"])
+    return {"name": w.name, "sizes": w.sizes, "dtype": w.dtype, "flops": w.flops, "algorithmic_bytes": w.bytes,
+            "kernel_us_mean": round(st["mean_ms"] * 1e3, 2), "kernel_us_median": round(st["median_ms"] * 1e3, 2),
+            "kernel_us_min": round(st["min_ms"] * 1e3, 2),
+            "gflops": round(w.flops / (st["mean_ms"] * 1e-3) / 1e9, 1),
+            "roofline": primary, "roofline_other": secondary,
+            "mapping": w.ex.info["spec"]}
+
+
+def cpu_baseline_and_verify(w, budget_s=20.0):
+    """Times the CPU oracle on a slab of the output (whole tensor when it fits the time budget) and
+    checks the GPU result on that slab.  Runs after ONE launch from a fresh C."""
+    import numpy as np
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import helpers
+    oracle = helpers.Oracle()
+    pkg_text = open(os.path.join(ROOT, "cgo2019-ae_amd", "expressions", w.plan_file)).read()
+    expr = helpers.parse_expression(pkg_text)
+    threads = min(oracle.max_threads(), 16)
+    last = w.sizes[len(expr["out_idx"]) - 1]
+    # probe one slice of the slowest output index to size the sample
+    probe = w.hC.copy()
+    t0 = time.perf_counter()
+    oracle.contract(expr, w.sizes, probe, w.hA, w.hB, threads=threads, last_range=(0, 1))
+    per_slice = time.perf_counter() - t0
+    n_slices = int(max(1, min(last, budget_s / max(per_slice, 1e-6))))
+    want = w.hC.copy()
+    t0 = time.perf_counter()
+    oracle.contract(expr, w.sizes, want, w.hA, w.hB, threads=threads, last_range=(0, n_slices))
+    cpu_s = time.perf_counter() - t0
+    frac = n_slices / last
+    slab = (w.nC // last) * n_slices
+    # one GPU launch from a fresh C
+    w.reset_c()
+    w.launch(0)
+    torch.cuda.synchronize()
+    got = w.dC[0].cpu().numpy()
+    err = helpers.rel_error(got[:slab], want[:slab])
+    w.reset_c()
+    base = {"value": round(w.flops * frac / cpu_s / 1e9, 2), "unit": "GFLOP/s", "cores": threads, "kind": "port",
+            "sample": "%d of %d slices of the slowest output index (%.0f%% of the contraction), %.2f s wall on %d threads"
+                      % (n_slices, last, 100 * frac, cpu_s, threads)}
+    verify = {"checked_elements": int(slab), "max_rel_err": err, "tolerance": TOL[w.dtype],
+              "definition": "|gpu-ref| / max(|ref|, rms(ref))", "pass": bool(err <= TOL[w.dtype])}
+    return base, verify
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only-headline", action="store_true", help="skip the table of the other BASELINE configs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
+    ap.add_argument("--workload", default=HEADLINE, help="expression object to use as the headline workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the contraction shards without "
+              "collectives, see DESIGN.md, but no multi-GPU path is built)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import cogent_mi355 as pkg
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    tools = pkg.HostTools()
+    driver = pkg.Driver()
+
+    entry = pkg.manifest_entry(args.workload)
+    w = Workload(pkg, tools, entry, entry["bench_sizes"])
+    w.plan_file = entry["file"]
+
+    cpu, verify = (None, None)
+    if not args.no_cpu:
+        cpu, verify = cpu_baseline_and_verify(w)
+
+    # ---- the timed region: W warm-up steps, then exactly K steps between two synchronisations
+    for i in range(args.warmup):
+        w.launch(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        w.launch(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    # ---- per-launch kernel durations from HIP events on the launch stream
+    head = time_workload(driver, w, args.warmup, args.steps)
+    head["roofline"]["traffic"] = read_traffic(w.name)
+
+    table = []
+    if not args.only_headline:
+        del w
+        torch.cuda.empty_cache()
+        for e in pkg.manifest():
+            if not e["name"].startswith("cfg"):
+                continue
+            for sizes in [e["bench_sizes"]] + e.get("alt_sizes", []):
+                wl = Workload(pkg, tools, e, sizes)
+                table.append(time_workload(driver, wl, 10, 50))
+                del wl
+                torch.cuda.empty_cache()
+
+    out = {
+        "metric": "GFLOP/s per contraction (fp64/fp32) + % MFMA peak or % HBM GB/s, 1 GPU",
+        "value": round(head["flops"] / (ms_per_step * 1e-3) / 1e9, 1),
+        "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: fp64 C[a,b,c,d] += sum_e A[a,e,b]*B[d,e,c], all extents 72 "
+                               "(column-major: %s)" % pkg.Expression(args.workload).expression.strip()
+                   if args.workload == HEADLINE else args.workload,
+                   "sizes": head["sizes"], "flops_per_step": head["flops"], "algorithmic_bytes_per_step": head["algorithmic_bytes"],
+                   "mapping": head["mapping"], "c_buffers_rotated": True},
+        "kernel_us_mean": head["kernel_us_mean"], "kernel_us_median": head["kernel_us_median"],
+        "roofline": head["roofline"], "roofline_other": head["roofline_other"],
+        "cpu_baseline": cpu, "verify": verify,
+        "all_configs": table,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
