@@ -160,7 +160,11 @@ __device__ __forceinline__ void slice_store(const typename Cfg::T (&reg)[SLOTS],
 // tile and the tile products need no padding; INT_FULL: the same for the
 // contracted indices.  (The reference picks among four kernels by the same two
 // tests, cogent/src/codes/kernels/tc_interface.py:1150-1175.)
-template <class Cfg, bool EXT_FULL, bool INT_FULL>
+//
+// ONE_KB: the whole contracted range fits one K block (every contracted extent <= its tile), the
+// shape of the HBM-bound many-index contractions.  The K loop, its odometer and the register
+// prefetch of the next slices disappear, which frees registers for more resident wavefronts.
+template <class Cfg, bool EXT_FULL, bool INT_FULL, bool ONE_KB>
 __global__ __launch_bounds__(Cfg::NT)
 void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __restrict__ X,
                     const typename Cfg::T* __restrict__ Y, const TcDims d)
@@ -177,9 +181,12 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     constexpr int LDS_X = lds_elems<OX, Cfg::BKP>();
     constexpr int LDS_Y = lds_elems<OY, Cfg::BKP>();
     constexpr bool PADDED = (Cfg::BKP != Cfg::BK) || (Cfg::BXP != Cfg::BX) || (Cfg::BYP != Cfg::BY);
+    // two LDS stages when there is a K loop and both fit the static 64 KB: the next slices are
+    // written while other wavefronts still read the current ones, one barrier per K block
+    constexpr int NBUF = (!ONE_KB && 2 * (LDS_X + LDS_Y) * (int)sizeof(T) <= 65536) ? 2 : 1;
 
-    __shared__ T lds_x[LDS_X];
-    __shared__ T lds_y[LDS_Y];
+    __shared__ T lds_x_all[NBUF * LDS_X];
+    __shared__ T lds_y_all[NBUF * LDS_Y];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -191,7 +198,15 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     int rem[Cfg::NIDX];
     int64_t baseC = 0, baseX = 0, baseY = 0;
     {
-        unsigned b = blockIdx.x;
+        // Workgroups are handed to the 8 XCDs round-robin and every XCD has its own L2: give XCD x
+        // a CONTIGUOUS range of output tiles, so that the tiles resident on one XCD share their
+        // operand panels in that L2.
+        unsigned b;
+        {
+            const unsigned n = d.nblocks, xcd = blockIdx.x % 8u, idx = blockIdx.x / 8u;
+            const unsigned q = n / 8u, r = n % 8u;
+            b = xcd * q + (xcd < r ? xcd : r) + idx;
+        }
 #pragma unroll
         for (int i = 0; i < Cfg::NX; i++) {
             const int id = Cfg::x_id(i);
@@ -269,8 +284,9 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 
     // ---- padding rows/columns of the LDS slices are never written by the staging: clear once
     if (PADDED) {
-        for (int i = tid; i < LDS_X; i += NT) lds_x[i] = (T)0;
-        for (int i = tid; i < LDS_Y; i += NT) lds_y[i] = (T)0;
+        for (int i = tid; i < NBUF * LDS_X; i += NT) lds_x_all[i] = (T)0;
+        for (int i = tid; i < NBUF * LDS_Y; i += NT) lds_y_all[i] = (T)0;
+        __syncthreads();
     }
 
     // ---- K loop
@@ -282,13 +298,24 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb, d, rem, tid);
     slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb, d, rem, tid);
 
-    for (int kb = 0; kb < d.nkb; kb++) {
-        __syncthreads();                       // previous slice fully consumed (and padding cleared)
-        slice_store<Cfg, OX, false>(rx, lds_x, d, tid);
-        slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y, d, tid);
+    const int nkb = ONE_KB ? 1 : d.nkb;
+    if (NBUF == 2) {
+        slice_store<Cfg, OX, false>(rx, lds_x_all, d, tid);
+        slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y_all, d, tid);
         __syncthreads();
+    }
+    for (int kb = 0; kb < nkb; kb++) {
+        T* lds_x = lds_x_all + (NBUF == 2 ? (kb & 1) * LDS_X : 0);
+        T* lds_y = lds_y_all + (NBUF == 2 ? (kb & 1) * LDS_Y : 0);
+        if (NBUF == 1) {
+            if (!ONE_KB) __syncthreads();      // previous slices fully consumed
+            slice_store<Cfg, OX, false>(rx, lds_x, d, tid);
+            slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y, d, tid);
+            __syncthreads();
+        }
 
-        if (kb + 1 < d.nkb) {
+        const bool more = !ONE_KB && (kb + 1 < nkb);
+        if (more) {
             // advance the K-block odometer (first composite K index fastest) and prefetch
             int64_t kx = 0, ky = 0;
             bool carry = true;
@@ -317,6 +344,14 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
             for (int ti = 0; ti < TY; ti++)
 #pragma unroll
                 for (int tj = 0; tj < TX; tj++) acc[ti][tj] = MM::mma(a[ti], b[tj], acc[ti][tj]);
+        }
+
+        if (NBUF == 2) {
+            if (more) {
+                slice_store<Cfg, OX, false>(rx, lds_x_all + ((kb + 1) & 1) * LDS_X, d, tid);
+                slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y_all + ((kb + 1) & 1) * LDS_Y, d, tid);
+            }
+            __syncthreads();
         }
     }
 

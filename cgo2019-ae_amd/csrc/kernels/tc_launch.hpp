@@ -130,10 +130,17 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     const T* y = (const T*)(Cfg::X_IS_A ? B : A);
     const dim3 g((unsigned)grid), b(Cfg::NT);
     tc_clear_hip_error();
-    if (ext_full && int_full)       hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true>),   g, b, 0, stream, c, x, y, d);
-    else if (ext_full)              hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false>),  g, b, 0, stream, c, x, y, d);
-    else if (int_full)              hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true>),  g, b, 0, stream, c, x, y, d);
-    else                            hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false>), g, b, 0, stream, c, x, y, d);
+    if (nkb == 1) {
+        if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, true>),    g, b, 0, stream, c, x, y, d);
+        else if (ext_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false, true>),   g, b, 0, stream, c, x, y, d);
+        else if (int_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true, true>),   g, b, 0, stream, c, x, y, d);
+        else                        hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false, true>),  g, b, 0, stream, c, x, y, d);
+    } else {
+        if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, false>),   g, b, 0, stream, c, x, y, d);
+        else if (ext_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false, false>),  g, b, 0, stream, c, x, y, d);
+        else if (int_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true, false>),  g, b, 0, stream, c, x, y, d);
+        else                        hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false, false>), g, b, 0, stream, c, x, y, d);
+    }
     return tc_check_launch("tiled kernel launch failed");
 }
 

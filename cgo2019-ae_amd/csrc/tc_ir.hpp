@@ -45,8 +45,8 @@ struct ArchGfx950 {
     int vgpr_per_lane = 512;                 // unified VGPR+AGPR file at one wave per SIMD
     double clock_hz = 2.4e9;
     double hbm_bytes_per_s = 8.0e12;         // published peak
-    double hbm_sustained_fraction = 0.70;    // what a plain copy kernel reaches on the part
-    double l2_bytes_per_s = 14.0e12;         // aggregate L2/Infinity-Cache rate for re-read operand slices
+    double hbm_sustained_fraction = 0.66;    // what a plain read-modify-write kernel reaches on the part
+    double l2_bytes_per_s = 10.0e12;         // aggregate L2/Infinity-Cache rate for re-read operand slices
     double lds_bytes_per_clk_cu = 128.0;
     double mfma_f64_flops = 78.6e12;
     double mfma_f32_flops = 157.3e12;

@@ -76,7 +76,10 @@ static std::vector<int> tile_options(int ext, int cap)
 
 struct SideCand { std::vector<int> ids, tiles; int B; };
 
-// greedy prefix: leading indices take their full extent, one index a partial tile, the rest 1
+// Tile lists for one side.  The reference's greedy prefix (leading indices at their full extent,
+// one index with a partial tile, the rest 1; enumeration.py:352-374) plus one generalisation:
+// the index after the partial one may carry a tile too, e.g. d:24,c:4 of extents 72,72, which
+// gives 96 = 6 MFMA tiles where the prefix rule only offers 72 (4.5 tiles) or 144.
 static void prefix_candidates(const Contraction& c, const std::vector<int>& order, int maxB,
                               std::vector<SideCand>& out)
 {
@@ -87,15 +90,21 @@ static void prefix_candidates(const Contraction& c, const std::vector<int>& orde
         const int ext = c.indices[order[p]].rep_size;
         for (int t : tile_options(ext, maxB)) {
             if (P * t > maxB) break;
-            SideCand sc;
-            sc.ids = order;
-            sc.tiles.assign(n, 1);
-            for (int j = 0; j < p; j++) sc.tiles[j] = c.indices[order[j]].rep_size;
-            sc.tiles[p] = t;
-            sc.B = (int)(P * t);
-            std::vector<int> key = sc.ids;
-            key.insert(key.end(), sc.tiles.begin(), sc.tiles.end());
-            if (seen.insert(key).second) out.push_back(sc);
+            std::vector<int> second = {1};
+            if (p + 1 < n && t < ext && t >= 8) second = tile_options(c.indices[order[p + 1]].rep_size, maxB);
+            for (int t2 : second) {
+                if (P * t * t2 > maxB) break;
+                SideCand sc;
+                sc.ids = order;
+                sc.tiles.assign(n, 1);
+                for (int j = 0; j < p; j++) sc.tiles[j] = c.indices[order[j]].rep_size;
+                sc.tiles[p] = t;
+                if (p + 1 < n) sc.tiles[p + 1] = t2;
+                sc.B = (int)(P * t * t2);
+                std::vector<int> key = sc.ids;
+                key.insert(key.end(), sc.tiles.begin(), sc.tiles.end());
+                if (seen.insert(key).second) out.push_back(sc);
+            }
         }
         P *= ext;
         if (P > maxB) break;
@@ -236,27 +245,49 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
         if (tl != c.indices[id].rep_size) break;
     }
     const double c_hbm_eff = std::min(1.0, chunk * s / 128.0);
+    // address span of the block's C tile relative to its volume: compact tiles keep DRAM pages and
+    // TLB entries busy with fewer blocks (measured: tiling the Y side in C's own index order beats
+    // the operand's order by 20-40% on the 6-D contractions)
+    double span = 1, vol = 1, strideC = 1;
+    for (int id : c.out_idx) {
+        const int tl = tile_of(id);
+        span += (tl - 1) * strideC;
+        vol *= tl;
+        strideC *= ext(id);
+    }
+    const double spread = 1.0 + 0.012 * std::log2(std::max(1.0, span / vol));
 
-    // resident blocks per CU
+    // ---- registers per lane, calibrated on hipcc's reports for this kernel: accumulators, one
+    // value register set per staged slice element, C offsets, MFMA operands and ~40 of
+    // bookkeeping; with a K loop the per-element addresses are hoisted out of it (two more each)
     const int W = m.WX * m.WY;
-    const int acc_regs = m.TX * m.TY * mi.NREG * (int)(s / 4);
-    const int slots = (int)std::ceil((double)m.BK * (m.BX + m.BY) / (64.0 * W));
-    const int regs = acc_regs + slots * (int)(s / 4) * 2 + (m.TX + m.TY) * (int)(s / 4) + 48;
+    const int r4 = (int)(s / 4);
+    const int acc_regs = m.TX * m.TY * mi.NREG * r4;
+    const int slots = (int)(std::ceil((double)m.BK * m.BX / (64.0 * W)) + std::ceil((double)m.BK * m.BY / (64.0 * W)));
+    int regs = acc_regs + 40 + slots * r4 + (m.TX + m.TY * mi.NREG) + (m.TX + m.TY) * r4;
+    if (nkb > 1) regs += 2 * slots;
+    const int reg_cap = std::min(512, arch.vgpr_per_lane / ceil_div(W, arch.simd_per_cu));
+    const double spill_penalty = regs > reg_cap ? 1.0 + 2.0 * (double)(regs - reg_cap) / reg_cap : 1.0;
     int waves_per_simd = std::max(1, std::min(8, arch.vgpr_per_lane / std::max(regs, 64)));
-    int r = std::min(arch.lds_bytes_per_cu / std::max(m.lds_bytes, 1), arch.max_waves_per_cu / W);
+    const bool two_stage = nkb > 1 && 2 * m.lds_bytes <= arch.lds_bytes_per_block;
+    const int lds_block = m.lds_bytes * (two_stage ? 2 : 1);
+    int r = std::min(arch.lds_bytes_per_cu / std::max(lds_block, 1), arch.max_waves_per_cu / W);
     r = std::min(r, std::max(1, waves_per_simd * arch.simd_per_cu / W));
     r = std::max(r, 1);
+    r = (int)std::min<long long>(r, std::max<long long>(1, ceil_div((int)std::min<long long>(nblocks, 1 << 30), arch.n_cu)));
     m.blocks_per_cu = r;
+    const double waves_simd = (double)(r * W) / arch.simd_per_cu;      // resident wavefronts per SIMD
 
+    // ---- HBM: a streaming kernel reaches the sustained rate only with about four resident
+    // wavefronts per SIMD in different phases (load C / contract / store C); measured 0.75 at two
     const double bw = arch.hbm_bytes_per_s * arch.hbm_sustained_fraction;
-    // bytes in flight needed to cover HBM latency: about 48 KB per CU
-    const double inflight = (double)r * m.BX * m.BY * s + (double)r * m.BK * (m.BX + m.BY) * s;
-    const double lat_scale = std::min(1.0, inflight / (48.0 * 1024.0));
-    m.t_hbm = ((nA + nB) * s + 2.0 * nC * s / c_hbm_eff) / (bw * lat_scale);
+    // (wavefronts of one block move in lock-step between barriers, so blocks count too)
+    const double occ_eff = std::min(1.0, 0.5 + 0.125 * waves_simd) * (r >= 3 ? 1.0 : r == 2 ? 0.93 : 0.85);
+    m.t_hbm = ((nA + nB) * s + 2.0 * nC * s * spread / c_hbm_eff) / (bw * occ_eff);
     const double l1_bw = 64.0 * arch.n_cu * arch.clock_hz;
     const double t_l1 = 2.0 * nC * s / (l1_bw * c_l1_eff);
 
-    // operand slices are re-read by every block that needs them; they mostly hit in L2 / Infinity Cache
+    // ---- operand slices are re-read by every block that needs them; they mostly hit in L2 / Infinity Cache
     const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
     const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
     auto op_eff = [&](const std::vector<int>& op) {
@@ -269,22 +300,28 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const double stage_y = (double)nblocks * nkb * m.BK * m.BY * s;
     m.t_l2 = stage_x / (arch.l2_bytes_per_s * op_eff(xop)) + stage_y / (arch.l2_bytes_per_s * op_eff(yop));
 
-    const double simd_busy = std::min(1.0, (double)(W * r) / (arch.simd_per_cu * std::ceil((double)(W * r) / arch.simd_per_cu)));
+    // ---- matrix cores: wavefronts of the resident blocks spread over 4 SIMDs (9 wavefronts leave
+    // three SIMDs idle a third of the time); every wavefront also pays about 700 issue cycles of
+    // address arithmetic, staging and barrier per K block next to its MFMAs
+    const double simd_busy = waves_simd / std::ceil(waves_simd);
     const double n_mfma = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * (m.BXP / mi.MT) * (m.BYP / mi.MT);
-    m.t_mfma = n_mfma * mi.cycles / (arch.n_cu * arch.simd_per_cu * arch.clock_hz) / simd_busy;
+    const double simd_hz = (double)arch.n_cu * arch.simd_per_cu * arch.clock_hz;
+    const double t_overhead = (double)nblocks * nkb * W * 700.0 / simd_hz;
+    m.t_mfma = (n_mfma * mi.cycles / simd_hz + t_overhead) / simd_busy;
 
     const double lds_reads = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * W * (m.TX + m.TY) * 64.0 * s;
     m.t_lds = (lds_reads + stage_x + stage_y) / (arch.lds_bytes_per_clk_cu * arch.n_cu * arch.clock_hz);
 
-    const double slots_total = (double)arch.n_cu * r;
-    const double rounds = std::ceil((double)nblocks / slots_total);
-    m.tail_eff = (double)nblocks / (rounds * slots_total);
+    // ---- tail: blocks are handed out as slots free up, so the last CU finishes at most one block late
+    const double per_cu = (double)nblocks / arch.n_cu;
+    m.tail_eff = per_cu / std::ceil(per_cu);
+    if (per_cu > 1.0) m.tail_eff = std::max(m.tail_eff, per_cu / (std::floor(per_cu) + 1.0));
 
-    const double parts[4] = {m.t_hbm + 0.0, m.t_l2, m.t_mfma, m.t_lds};
-    double mx = std::max(t_l1, 0.0), sum = t_l1;
+    const double parts[4] = {m.t_hbm, m.t_l2, m.t_mfma, m.t_lds};
+    double mx = t_l1, sum = t_l1;
     for (double p : parts) { mx = std::max(mx, p); sum += p; }
     // the slowest pipe sets the pace; the others overlap imperfectly
-    m.cost = (mx + 0.15 * (sum - mx)) / std::max(m.tail_eff, 0.05) + 2.0e-6;
+    m.cost = (mx + 0.15 * (sum - mx)) * spill_penalty / std::max(m.tail_eff, 0.05) + 2.0e-6;
 }
 
 static void wave_layouts(int nx, int ny, int max_acc_tiles, std::vector<std::array<int, 4>>& out)
@@ -338,8 +375,8 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
     }
 
     std::vector<SideCand> xc, yc, kc;
-    for (auto& o : x_orders) prefix_candidates(c, o, 512, xc);
-    for (auto& o : y_orders) prefix_candidates(c, o, 512, yc);
+    for (auto& o : x_orders) prefix_candidates(c, o, 256, xc);
+    for (auto& o : y_orders) prefix_candidates(c, o, 256, yc);
     for (auto& o : k_orders) prefix_candidates(c, o, 64, kc);
     // an input without external indices (matrix-vector shapes) or without a summed index: one empty tile
     if (yc.empty()) yc.push_back(SideCand{{}, {}, 1});
@@ -348,6 +385,16 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
     for (auto& s : xc) max_bx = std::max(max_bx, s.B);
     for (auto& s : yc) max_by = std::max(max_by, s.B);
     for (auto& s : kc) max_bk = std::max(max_bk, s.B);
+    // external tile products that are whole MFMA tiles (or the whole side when it is small),
+    // K tiles that are whole MFMA steps
+    auto keep_whole = [](std::vector<SideCand>& v, int gran, int mx) {
+        std::vector<SideCand> o;
+        for (auto& s : v) if (s.B % gran == 0 || s.B == mx) o.push_back(s);
+        if (!o.empty()) v.swap(o);
+    };
+    keep_whole(xc, 16, max_bx);
+    keep_whole(yc, 16, max_by);
+    keep_whole(kc, 4, max_bk);
 
     const std::vector<int> mis = (t == DType::F64) ? std::vector<int>{0} : std::vector<int>{1, 2};
     for (int miv : mis) {
@@ -358,11 +405,11 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
             for (const SideCand& sx : xc) {
                 if (sx.B < std::min(8, max_bx)) continue;
                 const int nx = ceil_div(sx.B, mi.MT);
-                if ((double)sx.B / (nx * mi.MT) < 0.7 && sx.B != max_bx) continue;
+                if ((double)sx.B / (nx * mi.MT) < 0.8 && sx.B != max_bx) continue;
                 for (const SideCand& sy : yc) {
                     if (sy.B < std::min(8, max_by)) continue;
                     const int ny = ceil_div(sy.B, mi.MT);
-                    if ((double)sy.B / (ny * mi.MT) < 0.7 && sy.B != max_by) continue;
+                    if ((double)sy.B / (ny * mi.MT) < 0.8 && sy.B != max_by) continue;
                     std::vector<std::array<int, 4>> wl;
                     wave_layouts(nx, ny, max_acc_tiles, wl);
                     for (auto& w : wl) {

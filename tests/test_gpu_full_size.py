@@ -1,0 +1,88 @@
+"""The BASELINE configurations at their FULL sizes, through properties that need no CPU pass over
+the whole tensor: a slab of the output against the CPU oracle, the whole output against the plain
+kernel (which is bit-exact with the oracle at the sizes test_gpu_parity.py covers), closed forms and
+linearity.  Tolerances: 1e-12 (fp64) / 1e-5 (fp32) on |gpu-ref| / max(|ref|, rms(ref))."""
+import numpy as np
+import pytest
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"f64": 1e-12, "f32": 1e-5}
+
+
+def configs():
+    import json
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "cgo2019-ae_amd", "expressions", "manifest.json")) as f:
+        return [(e["name"], e["bench_sizes"], e.get("c_init") == "seeded") for e in json.load(f)["expressions"]
+                if e["name"].startswith("cfg")]
+
+
+@pytest.mark.parametrize("name,sizes,seeded", configs(), ids=[c[0] for c in configs()])
+def test_full_size_against_plain_kernel_and_oracle_slab(name, sizes, seeded, tools, oracle):
+    import torch
+    import cogent_mi355 as pkg
+    ex = pkg.Expression(name)
+    expr = helpers.parse_expression(pkg.expression_text(name))
+    dtype = np.float64 if ex.dtype == "f64" else np.float32
+    nC, nA, nB = helpers.tensor_sizes(expr, sizes)
+    A = tools.fill_uniform(np.empty(nA, dtype), 1)
+    B = tools.fill_uniform(np.empty(nB, dtype), 2)
+    C = tools.fill_uniform(np.empty(nC, dtype), 3) if seeded else np.zeros(nC, dtype)
+    dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    d_tiled, d_plain = torch.from_numpy(C).cuda(), torch.from_numpy(C).cuda()
+    print("[gpu] full size %s %s" % (name, sizes), flush=True)
+    assert ex.entry(sizes, d_tiled.data_ptr(), dA.data_ptr(), dB.data_ptr()) == 0, ex.last_error()
+    assert ex.run(sizes, d_plain.data_ptr(), dA.data_ptr(), dB.data_ptr(), None, 1) == 0, ex.last_error()
+    torch.cuda.synchronize()
+    # whole tensor on the device: tiled MFMA kernel vs plain kernel
+    ref = d_plain.double()
+    rms = torch.sqrt(torch.mean(ref * ref)).item() or 1.0
+    err = (torch.abs(d_tiled.double() - ref) / torch.clamp(torch.abs(ref), min=rms)).max().item()
+    assert err <= TOL[ex.dtype], "tiled vs plain: %.3g" % err
+    # a slab of the slowest output index against the CPU oracle (a few hundred MFLOP at most)
+    last = sizes[len(expr["out_idx"]) - 1]
+    per_slice = 2.0 * np.prod(sizes, dtype=np.float64) / last
+    n = int(max(1, min(last, 4e8 // per_slice)))
+    want = oracle.contract(expr, sizes, C.copy(), A, B, last_range=(0, n))
+    slab = (nC // last) * n
+    got = d_tiled[:slab].cpu().numpy()
+    assert helpers.rel_error(got, want[:slab]) <= TOL[ex.dtype]
+    got_plain = d_plain[:slab].cpu().numpy()
+    assert np.array_equal(got_plain, want[:slab]), "plain kernel is not bit-exact with the oracle"
+
+
+@pytest.mark.parametrize("name", ["cfg2_f64", "cfg3_f64", "cfg4_16_f32", "cfg5_9_f64"])
+def test_full_size_closed_form_and_linearity(name, tools):
+    import torch
+    import cogent_mi355 as pkg
+    ex = pkg.Expression(name)
+    entry = pkg.manifest_entry(name)
+    sizes = entry["bench_sizes"]
+    expr = helpers.parse_expression(pkg.expression_text(name))
+    tdtype = torch.float64 if ex.dtype == "f64" else torch.float32
+    nC, nA, nB = helpers.tensor_sizes(expr, sizes)
+    ksize = int(np.prod(sizes[len(expr["out_idx"]):]))
+    print("[gpu] closed form %s" % name, flush=True)
+    # all ones: every output element equals the product of the contracted extents, exactly
+    ones_a = torch.ones(nA, dtype=tdtype, device="cuda")
+    ones_b = torch.ones(nB, dtype=tdtype, device="cuda")
+    c = torch.zeros(nC, dtype=tdtype, device="cuda")
+    assert ex.entry(sizes, c.data_ptr(), ones_a.data_ptr(), ones_b.data_ptr()) == 0
+    torch.cuda.synchronize()
+    assert bool((c == float(ksize)).all())
+    # linearity in A: scaling A by 2 scales the result by exactly 2 (power of two: no rounding)
+    np_dtype = np.float64 if ex.dtype == "f64" else np.float32
+    a = torch.from_numpy(tools.fill_uniform(np.empty(nA, np_dtype), 7)).cuda()
+    b = torch.from_numpy(tools.fill_uniform(np.empty(nB, np_dtype), 8)).cuda()
+    c1 = torch.zeros(nC, dtype=tdtype, device="cuda")
+    c2 = torch.zeros(nC, dtype=tdtype, device="cuda")
+    assert ex.entry(sizes, c1.data_ptr(), a.data_ptr(), b.data_ptr()) == 0
+    a2 = a * 2
+    assert ex.entry(sizes, c2.data_ptr(), a2.data_ptr(), b.data_ptr()) == 0
+    torch.cuda.synchronize()
+    assert bool((c2 == 2 * c1).all())
+    assert float(c1.abs().max()) > 0

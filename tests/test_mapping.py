@@ -1,0 +1,97 @@
+"""Invariants of the gfx950 index-to-tile mapping pass (the counterpart of the reference's
+enumeration + cost model + selection; no equality with the reference's pick is claimed, its
+mapping targets warp-32 CUDA).  Checked for every expression of the corpus in both element types."""
+import glob
+import os
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXPR_DIR = os.path.join(ROOT, "cgo2019-ae_amd", "expressions")
+FILES = sorted(glob.glob(os.path.join(EXPR_DIR, "*.in")))
+MT = {"v_mfma_f64_16x16x4_f64": (16, 4), "v_mfma_f32_16x16x4_f32": (16, 4), "v_mfma_f32_32x32x2_f32": (32, 2)}
+
+
+def check_mapping(info, m, dtype):
+    ext = dict(zip(info["out_idx"] + info["sum_idx"], info["rep_sizes"]))
+    x_op = info["a_idx"] if m["x_operand"] == info["a"] else info["b_idx"]
+    y_op = info["b_idx"] if m["x_operand"] == info["a"] else info["a_idx"]
+    xs, ys, ks = [n for n, _ in m["x"]], [n for n, _ in m["y"]], [n for n, _ in m["k"]]
+    # every index mapped exactly once, on the right side
+    assert sorted(xs + ys + ks) == sorted(ext)
+    assert set(xs) == {i for i in x_op if i in info["out_idx"]}
+    assert set(ys) == {i for i in y_op if i in info["out_idx"]}
+    assert set(ks) == set(info["sum_idx"])
+    # the X side is the input that holds the output's fastest index, and that index leads its tile list
+    assert info["out_idx"][0] in x_op and xs[0] == info["out_idx"][0]
+    mt, kstep = MT[m["mfma"]]
+    assert (dtype == "DOUBLE") == m["mfma"].startswith("v_mfma_f64")
+    prod = lambda side: eval("*".join(str(t) for _, t in side) or "1")
+    bx, by, bk = m["block_tile"]
+    assert (bx, by, bk) == (prod(m["x"]), prod(m["y"]), prod(m["k"]))
+    for name, t in m["x"] + m["y"] + m["k"]:
+        assert 1 <= t
+    px, py, pk = m["padded"]
+    wx, wy = m["waves"]
+    tx, ty = m["mfma_tiles_per_wave"]
+    assert px == wx * tx * mt >= bx and py == wy * ty * mt >= by and pk >= bk and pk % kstep == 0
+    assert m["threads"] == 64 * wx * wy and 64 <= m["threads"] <= 1024
+    assert m["lds_bytes"] <= 64 * 1024
+    blocks = 1
+    for name, t in m["x"] + m["y"]:
+        blocks *= -(-ext[name] // t)
+    assert m["model"]["blocks"] == blocks
+    ksteps = 1
+    for name, t in m["k"]:
+        ksteps *= -(-ext[name] // t)
+    assert m["model"]["k_steps"] == ksteps
+    assert m["model"]["cost_us"] > 0
+
+
+@pytest.mark.parametrize("path", FILES, ids=[os.path.basename(p) for p in FILES])
+@pytest.mark.parametrize("dtype", ["DOUBLE", "FLOAT"])
+def test_chosen_mapping_invariants(path, dtype, tools):
+    plan = tools.plan(open(path).read(), dtype)
+    check_mapping(plan.info, plan.info["mapping"], dtype)
+
+
+def test_candidates_are_sorted_and_admissible(tools):
+    plan = tools.plan(open(os.path.join(EXPR_DIR, "cfg5_3_f64.in")).read(), "DOUBLE")
+    cands = plan.candidates(200)
+    assert len(cands) > 20
+    costs = [c["model"]["cost_us"] for c in cands]
+    assert costs == sorted(costs)
+    for c in cands:
+        check_mapping(plan.info, c, "DOUBLE")
+    assert cands[0]["spec"] == plan.info["mapping"]["spec"]
+
+
+def test_manual_rank_and_spec_round_trip(tools):
+    text = open(os.path.join(EXPR_DIR, "cfg2_f64.in")).read()
+    auto = tools.plan(text, "DOUBLE")
+    cands = auto.candidates(5)
+    third = tools.plan(text, "DOUBLE", config_rank=2)          # the reference's manual pick
+    assert third.info["mapping"]["spec"] == cands[2]["spec"]
+    same = tools.plan(text, "DOUBLE", mapping_spec=cands[2]["spec"])
+    assert same.info["mapping"] == third.info["mapping"]
+    named = tools.plan(text, "DOUBLE", mapping_spec="x=d:24,c:4;y=b:24,a:4;k=e:8;w=2x2;t=3x3")
+    assert named.info["mapping"]["block_tile"] == [96, 96, 8] and named.info["mapping"]["threads"] == 256
+
+
+BAD_SPECS = [
+    "x=d:24;y=b:24,a:4;k=e:8;w=2x2;t=3x3",                # c unmapped
+    "x=d:24,c:4,b:2;y=a:4;k=e:8;w=2x2;t=3x3",             # b on the wrong side
+    "x=d:24,c:4;y=b:24,a:4;k=e:8;w=8x8;t=1x1",            # 4096 threads
+    "x=d:72,c:8;y=b:72,a:8;k=e:72;w=4x4;t=9x9",           # LDS and registers
+    "x=d:24,c:4;y=b:24,a:4;k=e:8;w=2x2;t=3x3;mi=1",       # fp32 instruction for fp64 data
+    "x=d:24,c:4;y=b:24,a:4;k=e:8;w=1x1;t=1x1",            # wavefront tiling smaller than the block tile
+]
+
+
+@pytest.mark.parametrize("spec", BAD_SPECS)
+def test_impossible_mappings_are_rejected(spec, tools):
+    import cogent_mi355
+    text = open(os.path.join(EXPR_DIR, "cfg2_f64.in")).read()
+    with pytest.raises(cogent_mi355.CogentError) as e:
+        tools.plan(text, "DOUBLE", mapping_spec=spec)
+    assert e.value.code == 3
