@@ -102,10 +102,10 @@ __device__ __forceinline__ int lds_addr(int k, int e) { return Op::LAY == 0 ? k 
 // lies inside the tensor.  rem[id] = extent[id] - tile origin along id.
 template <class Op, bool EXT_FULL, bool INT_FULL>
 __device__ __forceinline__ void slice_element(unsigned q, const TcDims& d, const int* rem,
-                                              int& goff, int& loff, bool& valid)
+                                              unsigned& goff, int& loff, bool& valid)
 {
     int e = 0, k = 0;
-    goff = 0;
+    goff = 0u;
     valid = true;
 #pragma unroll
     for (int j = 0; j < Op::R; j++) {
@@ -113,7 +113,7 @@ __device__ __forceinline__ void slice_element(unsigned q, const TcDims& d, const
         const int i = (int)(q % t);
         q /= t;
         const int id = Op::id(j);
-        goff += i * Op::stride(d, id);
+        goff += (unsigned)i * (unsigned)Op::stride(d, id);
         if (Op::isk(j)) {
             k += i * Op::mul(j);
             if (!INT_FULL) valid = valid && (i < rem[id]);
@@ -134,10 +134,10 @@ __device__ __forceinline__ void slice_load(typename Cfg::T (&reg)[SLOTS], const 
 #pragma unroll
     for (int s = 0; s < SLOTS; s++) {
         const unsigned q = (unsigned)tid + (unsigned)s * Cfg::NT;
-        int goff, loff; bool valid;
+        unsigned goff; int loff; bool valid;
         slice_element<Op, EXT_FULL, INT_FULL>(q, d, rem, goff, loff, valid);
         T v = (T)0;
-        if ((E % Cfg::NT == 0 || q < E) && valid) v = src[goff];
+        if ((E % Cfg::NT == 0 || q < E) && valid) v = *(const T*)((const char*)src + goff * (unsigned)sizeof(T));
         reg[s] = v;
     }
 }
@@ -150,9 +150,51 @@ __device__ __forceinline__ void slice_store(const typename Cfg::T (&reg)[SLOTS],
 #pragma unroll
     for (int s = 0; s < SLOTS; s++) {
         const unsigned q = (unsigned)tid + (unsigned)s * Cfg::NT;
-        int goff, loff; bool valid;
+        unsigned goff; int loff; bool valid;
         slice_element<Op, true, true>(q, d, nullptr, goff, loff, valid);
         if (E % Cfg::NT == 0 || q < E) lds[loff] = NEGATE ? -reg[s] : reg[s];
+    }
+}
+
+// Element offsets, relative to the block's C tile origin, of the accumulator elements a lane holds:
+// cx[tj] for its column in MFMA tile column tj, cy[ti][r] for the row of register r in tile row ti;
+// -1 marks positions outside the tensor (ragged tiles, padding).
+template <class Cfg, bool EXT_FULL>
+__device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const int* rem, const TcDims& d,
+                                               int (&cx)[Cfg::TX], int (&cy)[Cfg::TY][Mfma<Cfg::MI>::NREG])
+{
+    typedef Mfma<Cfg::MI> MM;
+    constexpr int MT = MM::MT, NREG = MM::NREG, TX = Cfg::TX, TY = Cfg::TY;
+#pragma unroll
+    for (int tj = 0; tj < TX; tj++) {
+        const int x = (wx * TX + tj) * MT + lane % MT;
+        unsigned q = (unsigned)x;
+        int off = 0; bool ok = (Cfg::BXP == Cfg::BX) || (x < Cfg::BX);
+#pragma unroll
+        for (int i = 0; i < Cfg::NX; i++) {
+            const int c = (int)(q % (unsigned)Cfg::x_tile(i));
+            q /= (unsigned)Cfg::x_tile(i);
+            off += c * d.sC[Cfg::x_id(i)];
+            if (!EXT_FULL) ok = ok && (c < rem[Cfg::x_id(i)]);
+        }
+        cx[tj] = ok ? off : -1;
+    }
+#pragma unroll
+    for (int ti = 0; ti < TY; ti++) {
+#pragma unroll
+        for (int r = 0; r < NREG; r++) {
+            const int y = (wy * TY + ti) * MT + MM::row(r, lane);
+            unsigned q = (unsigned)y;
+            int off = 0; bool ok = (Cfg::BYP == Cfg::BY) || (y < Cfg::BY);
+#pragma unroll
+            for (int i = 0; i < Cfg::NY; i++) {
+                const int c = (int)(q % (unsigned)Cfg::y_tile(i));
+                q /= (unsigned)Cfg::y_tile(i);
+                off += c * d.sC[Cfg::y_id(i)];
+                if (!EXT_FULL) ok = ok && (c < rem[Cfg::y_id(i)]);
+            }
+            cy[ti][r] = ok ? off : -1;
+        }
     }
 }
 
@@ -237,37 +279,7 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     // ---- where this lane's accumulator elements live in C (-1: outside)
     int cx[TX];
     int cy[TY][NREG];
-#pragma unroll
-    for (int tj = 0; tj < TX; tj++) {
-        const int x = (wx * TX + tj) * MT + lane % MT;
-        unsigned q = (unsigned)x;
-        int off = 0; bool ok = (Cfg::BXP == Cfg::BX) || (x < Cfg::BX);
-#pragma unroll
-        for (int i = 0; i < Cfg::NX; i++) {
-            const int c = (int)(q % (unsigned)Cfg::x_tile(i));
-            q /= (unsigned)Cfg::x_tile(i);
-            off += c * d.sC[Cfg::x_id(i)];
-            if (!EXT_FULL) ok = ok && (c < rem[Cfg::x_id(i)]);
-        }
-        cx[tj] = ok ? off : -1;
-    }
-#pragma unroll
-    for (int ti = 0; ti < TY; ti++) {
-#pragma unroll
-        for (int r = 0; r < NREG; r++) {
-            const int y = (wy * TY + ti) * MT + MM::row(r, lane);
-            unsigned q = (unsigned)y;
-            int off = 0; bool ok = (Cfg::BYP == Cfg::BY) || (y < Cfg::BY);
-#pragma unroll
-            for (int i = 0; i < Cfg::NY; i++) {
-                const int c = (int)(q % (unsigned)Cfg::y_tile(i));
-                q /= (unsigned)Cfg::y_tile(i);
-                off += c * d.sC[Cfg::y_id(i)];
-                if (!EXT_FULL) ok = ok && (c < rem[Cfg::y_id(i)]);
-            }
-            cy[ti][r] = ok ? off : -1;
-        }
-    }
+    c_tile_offsets<Cfg, EXT_FULL>(lane, wx, wy, rem, d, cx, cy);
 
     // ---- accumulators start from the C tile: C_in + sum, summed in k order
     Acc acc[TY][TX];
@@ -278,7 +290,7 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
             for (int r = 0; r < NREG; r++) {
                 T v = (T)0;
-                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) v = Cb[cx[tj] + cy[ti][r]];
+                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) v = *(const T*)((const char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
                 acc[ti][tj][r] = v;
             }
 
@@ -299,6 +311,13 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb, d, rem, tid);
 
     const int nkb = ONE_KB ? 1 : d.nkb;
+    if (!ONE_KB) {
+        // Drain the C-tile and first-slice loads BEFORE the K loop.  Otherwise the compiler has to
+        // assume, on every trip, that the accumulators may still be in flight, and its wait for
+        // them (an in-order counter) also waits for the prefetch issued at the top of the trip,
+        // which takes the prefetch's whole latency out of hiding.  s_waitcnt vmcnt(0).
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
     if (NBUF == 2) {
         slice_store<Cfg, OX, false>(rx, lds_x_all, d, tid);
         slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y_all, d, tid);
@@ -355,14 +374,21 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         }
     }
 
-    // ---- write the tile back
+    // ---- write the tile back.  With a K loop the offsets are derived again here from an opaque
+    // copy of the lane id instead of being kept in registers across the loop (one register per
+    // accumulator element otherwise, which costs a resident wavefront per SIMD).
+    if (!ONE_KB) {
+        int lane2 = lane;
+        asm volatile("" : "+v"(lane2));
+        c_tile_offsets<Cfg, EXT_FULL>(lane2, wx, wy, rem, d, cx, cy);
+    }
 #pragma unroll
     for (int ti = 0; ti < TY; ti++)
 #pragma unroll
         for (int tj = 0; tj < TX; tj++)
 #pragma unroll
             for (int r = 0; r < NREG; r++)
-                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) Cb[cx[tj] + cy[ti][r]] = acc[ti][tj][r];
+                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) *(T*)((char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T)) = acc[ti][tj][r];
 }
 
 // ---------------------------------------------------------------------------
