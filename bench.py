@@ -157,6 +157,9 @@ def main():
     ap.add_argument("--only-headline", action="store_true", help="skip the table of the other BASELINE configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
     ap.add_argument("--workload", default=HEADLINE, help="expression object to use as the headline workload")
+    ap.add_argument("--copy-only", type=int, default=0, metavar="BYTES",
+                    help="only run the plain device-to-device copy kernel on BYTES bytes, --steps times "
+                         "(the known-size yardstick the FETCH_SIZE / WRITE_SIZE counter readings are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the contraction shards without "
@@ -170,6 +173,14 @@ def main():
         sys.exit(1)
     tools = pkg.HostTools()
     driver = pkg.Driver()
+
+    if args.copy_only:
+        src = torch.ones(args.copy_only // 8, dtype=torch.float64, device="cuda")
+        dst = torch.zeros(args.copy_only // 8, dtype=torch.float64, device="cuda")
+        ms = driver.time_copy(src.data_ptr(), dst.data_ptr(), args.copy_only, args.warmup, args.steps)
+        print(json.dumps({"copy_bytes": args.copy_only, "ms_per_copy": ms,
+                          "GBps_read_plus_write": round(2 * args.copy_only / ms / 1e6, 1)}))
+        return
 
     entry = pkg.manifest_entry(args.workload)
     w = Workload(pkg, tools, entry, entry["bench_sizes"])

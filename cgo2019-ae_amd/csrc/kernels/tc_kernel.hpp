@@ -43,6 +43,7 @@ struct TcDims {
     int sY[TC_MAXI];     // element stride inside the Y-side operand
     int nkb;             // number of K blocks = product of nblk over contracted ids
     unsigned nblocks;    // number of output tiles = grid size
+    unsigned nxt;        // number of tiles along the composite X coordinate (product of nblk over X ids)
 };
 
 typedef double v4f64 __attribute__((ext_vector_type(4)));
@@ -248,6 +249,18 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
             const unsigned n = d.nblocks, xcd = blockIdx.x % 8u, idx = blockIdx.x / 8u;
             const unsigned q = n / 8u, r = n % 8u;
             b = xcd * q + (xcd < r ? xcd : r) + idx;
+        }
+        // Within that range walk the tile grid in bands of TILE_GROUP X-tiles (X fastest inside a
+        // band, then Y): the ~100 tiles in flight on an XCD then touch a dozen X panels and a dozen
+        // Y panels instead of every X panel, and the panels stay in the 4 MB L2 while C streams by.
+        {
+            constexpr unsigned GX = 8;
+            const unsigned nyt = d.nblocks / d.nxt;
+            const unsigned G = GX * nyt;
+            const unsigned g = b / G, r = b % G;
+            const unsigned first = g * GX;
+            const unsigned gx = (d.nxt - first) < GX ? (d.nxt - first) : GX;
+            b = (first + r % gx) + (r / gx) * d.nxt;
         }
 #pragma unroll
         for (int i = 0; i < Cfg::NX; i++) {

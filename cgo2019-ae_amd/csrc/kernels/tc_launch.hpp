@@ -110,6 +110,7 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
         d.nblk[id] = (sizes[id] + t - 1) / t; grid *= d.nblk[id];
         if (sizes[id] % t) ext_full = false;
     }
+    const int64_t nxt = grid;
     for (int i = 0; i < Cfg::NY; i++) {
         const int id = Cfg::y_id(i), t = Cfg::y_tile(i);
         d.nblk[id] = (sizes[id] + t - 1) / t; grid *= d.nblk[id];
@@ -124,6 +125,7 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     if (grid > lim || nkb > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
     d.nkb = (int)nkb;
     d.nblocks = (unsigned)grid;
+    d.nxt = (unsigned)nxt;
 
     T* c = (T*)C;
     const T* x = (const T*)(Cfg::X_IS_A ? A : B);
