@@ -238,6 +238,8 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     const int wy = wave / Cfg::WX;
 
     // ---- which output tile: X-side tiles vary fastest over the grid
+    constexpr int SK = ONE_KB ? 1 : Cfg::SK;
+    unsigned ks = 0;
     int rem[Cfg::NIDX];
     int64_t baseC = 0, baseX = 0, baseY = 0;
     {
@@ -250,12 +252,14 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
             const unsigned q = n / 8u, r = n % 8u;
             b = xcd * q + (xcd < r ? xcd : r) + idx;
         }
+        // split K: SK consecutive workgroups share one output tile, each takes a share of the K blocks
+        if (SK > 1) { ks = b % (unsigned)SK; b /= (unsigned)SK; }
         // Within that range walk the tile grid in bands of TILE_GROUP X-tiles (X fastest inside a
         // band, then Y): the ~100 tiles in flight on an XCD then touch a dozen X panels and a dozen
         // Y panels instead of every X panel, and the panels stay in the 4 MB L2 while C streams by.
         {
             constexpr unsigned GX = 8;
-            const unsigned nyt = d.nblocks / d.nxt;
+            const unsigned nyt = (d.nblocks / (unsigned)SK) / d.nxt;
             const unsigned G = GX * nyt;
             const unsigned g = b / G, r = b % G;
             const unsigned first = g * GX;
@@ -303,7 +307,7 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
             for (int r = 0; r < NREG; r++) {
                 T v = (T)0;
-                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) v = *(const T*)((const char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
+                if (SK == 1 && ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0))) v = *(const T*)((const char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
                 acc[ti][tj][r] = v;
             }
 
@@ -318,12 +322,30 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     int kbc[Cfg::NK > 0 ? Cfg::NK : 1];
 #pragma unroll
     for (int i = 0; i < Cfg::NK; i++) kbc[i] = 0;
+    // this workgroup's share of the K blocks: [kb0, kb0 + nkb)
+    int kb0 = 0, nkb = ONE_KB ? 1 : d.nkb;
+    int64_t kx0 = 0, ky0 = 0;
+    if (SK > 1) {
+        kb0 = (int)(((int64_t)ks * d.nkb) / SK);
+        nkb = (int)(((int64_t)(ks + 1) * d.nkb) / SK) - kb0;
+        if (nkb <= 0) return;                      // more splits than K blocks: uniform for the block
+        unsigned q = (unsigned)kb0;
+#pragma unroll
+        for (int i = 0; i < Cfg::NK; i++) {
+            const int id = Cfg::k_id(i);
+            kbc[i] = (int)(q % (unsigned)d.nblk[id]);
+            q /= (unsigned)d.nblk[id];
+            const int o = kbc[i] * Cfg::k_tile(i);
+            rem[id] = d.ext[id] - o;
+            kx0 += (int64_t)o * d.sX[id];
+            ky0 += (int64_t)o * d.sY[id];
+        }
+    }
 
     T rx[SLOTS_X], ry[SLOTS_Y];
-    slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb, d, rem, tid);
-    slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb, d, rem, tid);
+    slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb + kx0, d, rem, tid);
+    slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb + ky0, d, rem, tid);
 
-    const int nkb = ONE_KB ? 1 : d.nkb;
     if (!ONE_KB) {
         // Drain the C-tile and first-slice loads BEFORE the K loop.  Otherwise the compiler has to
         // assume, on every trip, that the accumulators may still be in flight, and its wait for
@@ -401,7 +423,11 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         for (int tj = 0; tj < TX; tj++)
 #pragma unroll
             for (int r = 0; r < NREG; r++)
-                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) *(T*)((char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T)) = acc[ti][tj][r];
+                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) {
+                    T* dst = (T*)((char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
+                    if (SK == 1) *dst = acc[ti][tj][r];
+                    else unsafeAtomicAdd(dst, acc[ti][tj][r]);   // hardware global_atomic_add, device scope
+                }
 }
 
 // ---------------------------------------------------------------------------

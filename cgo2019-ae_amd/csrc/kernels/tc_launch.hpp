@@ -124,6 +124,10 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     }
     if (grid > lim || nkb > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
     d.nkb = (int)nkb;
+    // split K only when there is a K loop to split; the single-K-block kernels ignore Cfg::SK
+    const int sk = (nkb == 1) ? 1 : Cfg::SK;
+    grid *= sk;
+    if (grid > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
     d.nblocks = (unsigned)grid;
     d.nxt = (unsigned)nxt;
 

@@ -64,6 +64,7 @@ struct Mapping {
     int BXP = 0, BYP = 0, BKP = 0;            // padded to MFMA granularity
     int WX = 1, WY = 1, TX = 1, TY = 1;       // wavefront grid and MFMA tiles per wavefront
     int MI = 0;                               // 0 f64 16x16x4, 1 f32 16x16x4, 2 f32 32x32x2
+    int SK = 1;                               // split-K factor: SK workgroups per output tile, atomic accumulate
     int layx = 0, ldx = 0, layy = 0, ldy = 0; // LDS layout per operand
     // model outputs
     double t_hbm = 0, t_l2 = 0, t_mfma = 0, t_lds = 0, tail_eff = 1, cost = 0;

@@ -62,6 +62,7 @@ std::string Mapping::spec() const
     side("k", k_ids, k_tiles);
     o << "w=" << WX << "x" << WY << ";t=" << TX << "x" << TY << ";mi=" << MI
       << ";lx=" << layx << ";ly=" << layy;
+    if (SK > 1) o << ";sk=" << SK;
     return o.str();
 }
 
@@ -196,6 +197,7 @@ bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const 
     const int reg_budget = std::min(512, arch.vgpr_per_lane / waves_per_simd);
     if (acc_regs > 256 || acc_regs * 2 > reg_budget) { err = "accumulator tiles exceed the register budget per lane"; return false; }
     if (m.layx < 0 || m.layx > 1 || m.layy < 0 || m.layy > 1) { err = "unknown LDS layout"; return false; }
+    if (m.SK < 1 || m.SK > 64) { err = "split-K factor outside 1..64"; return false; }
     return true;
 }
 
@@ -221,6 +223,11 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     for (size_t i = 0; i < m.y_ids.size(); i++) nblocks *= ceil_div(c.indices[m.y_ids[i]].rep_size, m.y_tiles[i]);
     long long nkb = 1;
     for (size_t i = 0; i < m.k_ids.size(); i++) nkb *= ceil_div(c.indices[m.k_ids[i]].rep_size, m.k_tiles[i]);
+    // split K: SK workgroups per tile, each a share of the K blocks, accumulated with atomics
+    const int sk = (nkb > 1) ? std::max(1, m.SK) : 1;
+    const double c_passes = sk > 1 ? (double)sk : 1.0;
+    nblocks *= sk;
+    nkb = (nkb + sk - 1) / sk;
     m.n_blocks = nblocks;
     m.steps_main_loop = (int)nkb;
 
@@ -283,9 +290,9 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const double bw = arch.hbm_bytes_per_s * arch.hbm_sustained_fraction;
     // (wavefronts of one block move in lock-step between barriers, so blocks count too)
     const double occ_eff = std::min(1.0, 0.5 + 0.125 * waves_simd) * (r >= 3 ? 1.0 : r == 2 ? 0.93 : 0.85);
-    m.t_hbm = ((nA + nB) * s + 2.0 * nC * s * spread / c_hbm_eff) / (bw * occ_eff);
+    m.t_hbm = ((nA + nB) * s + 2.0 * nC * s * c_passes * spread / c_hbm_eff) / (bw * occ_eff);
     const double l1_bw = 64.0 * arch.n_cu * arch.clock_hz;
-    const double t_l1 = 2.0 * nC * s / (l1_bw * c_l1_eff);
+    const double t_l1 = 2.0 * nC * s * c_passes / (l1_bw * c_l1_eff);
 
     // ---- operand slices are re-read by every block that needs them; they mostly hit in L2 / Infinity Cache
     const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
@@ -303,7 +310,10 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     // ---- matrix cores: wavefronts of the resident blocks spread over 4 SIMDs (9 wavefronts leave
     // three SIMDs idle a third of the time); every wavefront also pays about 700 issue cycles of
     // address arithmetic, staging and barrier per K block next to its MFMAs
-    const double simd_busy = waves_simd / std::ceil(waves_simd);
+    // (a block's wavefronts are dealt to the SIMDs starting at SIMD 0: 6 or 9 of them load the SIMDs unevenly;
+    // measured: 6-wavefront blocks run 40% slower than 4-wavefront ones on the same tile volume)
+    const double per_block = W >= arch.simd_per_cu ? ((double)W / arch.simd_per_cu) / std::ceil((double)W / arch.simd_per_cu) : 1.0;
+    const double simd_busy = std::min(waves_simd / std::ceil(waves_simd), per_block);
     const double n_mfma = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * (m.BXP / mi.MT) * (m.BYP / mi.MT);
     const double simd_hz = (double)arch.n_cu * arch.simd_per_cu * arch.clock_hz;
     const double t_overhead = (double)nblocks * nkb * W * 700.0 / simd_hz;
@@ -428,6 +438,15 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
                         if (!check_mapping(c, t, arch, m, err)) continue;
                         cost_model(c, t, arch, m);
                         out.push_back(m);
+                        // few output tiles and a long K loop: also try splitting K over 2, 4, 8 workgroups
+                        const long long tiles = m.n_blocks;
+                        const int ksteps = m.steps_main_loop;
+                        for (int sk = 2; sk <= 8 && tiles < 8LL * arch.n_cu && ksteps >= 8 * sk; sk *= 2) {
+                            Mapping ms = m;
+                            ms.SK = sk;
+                            cost_model(c, t, arch, ms);
+                            out.push_back(ms);
+                        }
                     }
                 }
             }
@@ -490,6 +509,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
             if (sscanf(val.c_str(), "%dx%d", &a, &b) != 2 || a < 1 || b < 1) { err = "mapping spec: bad " + key; return false; }
             if (key == "w") { m.WX = a; m.WY = b; } else { m.TX = a; m.TY = b; }
         } else if (key == "mi") m.MI = atoi(val.c_str());
+        else if (key == "sk") m.SK = atoi(val.c_str());
         else if (key == "lx") lx = atoi(val.c_str());
         else if (key == "ly") ly = atoi(val.c_str());
         else { err = "mapping spec: unknown key " + key; return false; }
@@ -522,7 +542,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

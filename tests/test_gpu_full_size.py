@@ -84,5 +84,11 @@ def test_full_size_closed_form_and_linearity(name, tools):
     a2 = a * 2
     assert ex.entry(sizes, c2.data_ptr(), a2.data_ptr(), b.data_ptr()) == 0
     torch.cuda.synchronize()
-    assert bool((c2 == 2 * c1).all())
+    if ex.info.get("split_k", 1) > 1:
+        # the K shares of a tile are added with atomics in arrival order: equal up to rounding only
+        rms = float(torch.sqrt(torch.mean(c1 * c1)))
+        err = float((torch.abs(c2 - 2 * c1) / torch.clamp(torch.abs(2 * c1), min=2 * rms)).max())
+        assert err <= TOL[ex.dtype]
+    else:
+        assert bool((c2 == 2 * c1).all())
     assert float(c1.abs().max()) > 0
