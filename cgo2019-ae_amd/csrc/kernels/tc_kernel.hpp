@@ -29,6 +29,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace cogent {
 
@@ -90,6 +91,16 @@ template <class Cfg> struct Operand<Cfg, 1> {
     __device__ static __forceinline__ constexpr int mul(int j)  { return Cfg::yo_mul(j); }
     __device__ static __forceinline__ int stride(const TcDims& d, int id) { return d.sY[id]; }
 };
+
+// A value that is the same in every lane, moved into scalar registers.  64-bit products of
+// uniform values are computed on the vector ALU (the scalar ALU has no 64-bit multiply) and would
+// otherwise stay in vector registers, which turns every address built from them into vector adds.
+__device__ __forceinline__ int64_t uniform64(int64_t v)
+{
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)(uint64_t)v);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
 
 template <class Op, int BKP>
 constexpr int lds_elems() { return Op::LAY == 0 ? BKP * Op::LD : Op::BEP * Op::LD; }
@@ -208,7 +219,7 @@ __device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const i
 // shape of the HBM-bound many-index contractions.  The K loop, its odometer and the register
 // prefetch of the next slices disappear, which frees registers for more resident wavefronts.
 template <class Cfg, bool EXT_FULL, bool INT_FULL, bool ONE_KB>
-__global__ __launch_bounds__(Cfg::NT)
+__global__ __launch_bounds__(Cfg::NT, Cfg::MINW)     // MINW: wavefronts per SIMD the register allocator must leave room for
 void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __restrict__ X,
                     const typename Cfg::T* __restrict__ Y, const TcDims d)
 {
@@ -289,16 +300,22 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
         for (int i = 0; i < Cfg::NK; i++) rem[Cfg::k_id(i)] = d.ext[Cfg::k_id(i)];
     }
-    T* __restrict__ Cb = C + baseC;
-    const T* __restrict__ Xb = X + baseX;
-    const T* __restrict__ Yb = Y + baseY;
+    T* __restrict__ Cb = C + uniform64(baseC);
+    const T* __restrict__ Xb = X + uniform64(baseX);
+    const T* __restrict__ Yb = Y + uniform64(baseY);
 
     // ---- where this lane's accumulator elements live in C (-1: outside)
     int cx[TX];
     int cy[TY][NREG];
     c_tile_offsets<Cfg, EXT_FULL>(lane, wx, wy, rem, d, cx, cy);
 
-    // ---- accumulators start from the C tile: C_in + sum, summed in k order
+    // ---- accumulators start from the C tile: C_in + sum, summed in k order.
+    // LATE_C: they start from zero instead and the C tile is loaded into registers of its own during
+    // the first trip of the K loop, AFTER that trip's prefetch was issued (loads return in order, so
+    // the wait for the prefetch does not wait for C): the block starts contracting one L2 latency
+    // after launch instead of one HBM latency, and the C read hides behind its own K loop.
+    constexpr bool LATE_C = !ONE_KB && SK == 1 && (Cfg::LATEC != 0);
+    Acc cpre[LATE_C ? TY : 1][LATE_C ? TX : 1];
     Acc acc[TY][TX];
 #pragma unroll
     for (int ti = 0; ti < TY; ti++)
@@ -307,7 +324,7 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
             for (int r = 0; r < NREG; r++) {
                 T v = (T)0;
-                if (SK == 1 && ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0))) v = *(const T*)((const char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
+                if (SK == 1 && !LATE_C && ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0))) v = *(const T*)((const char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
                 acc[ti][tj][r] = v;
             }
 
@@ -343,8 +360,8 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     }
 
     T rx[SLOTS_X], ry[SLOTS_Y];
-    slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb + kx0, d, rem, tid);
-    slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb + ky0, d, rem, tid);
+    slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb + uniform64(kx0), d, rem, tid);
+    slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb + uniform64(ky0), d, rem, tid);
 
     if (!ONE_KB) {
         // Drain the C-tile and first-slice loads BEFORE the K loop.  Otherwise the compiler has to
@@ -358,7 +375,7 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y_all, d, tid);
         __syncthreads();
     }
-    for (int kb = 0; kb < nkb; kb++) {
+    auto k_block = [&](const int kb, auto first_trip) {
         T* lds_x = lds_x_all + (NBUF == 2 ? (kb & 1) * LDS_X : 0);
         T* lds_y = lds_y_all + (NBUF == 2 ? (kb & 1) * LDS_Y : 0);
         if (NBUF == 1) {
@@ -382,8 +399,21 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
                 kx += (int64_t)o * d.sX[id];
                 ky += (int64_t)o * d.sY[id];
             }
-            slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb + kx, d, rem, tid);
-            slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb + ky, d, rem, tid);
+            slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb + uniform64(kx), d, rem, tid);
+            slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb + uniform64(ky), d, rem, tid);
+        }
+        if (LATE_C && decltype(first_trip)::value) {
+#pragma unroll
+            for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+                for (int tj = 0; tj < TX; tj++)
+#pragma unroll
+                    for (int r = 0; r < NREG; r++) {
+                        T v = (T)0;
+                        if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0))
+                            v = *(const T*)((const char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
+                        cpre[LATE_C ? ti : 0][LATE_C ? tj : 0][r] = v;
+                    }
         }
 
 #pragma unroll
@@ -407,7 +437,10 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
             }
             __syncthreads();
         }
-    }
+    };
+    // the first trip is a copy of its own so that what is in flight during it is known exactly
+    k_block(0, std::true_type());
+    for (int kb = 1; kb < nkb; kb++) k_block(kb, std::false_type());
 
     // ---- write the tile back.  With a K loop the offsets are derived again here from an opaque
     // copy of the lane id instead of being kept in registers across the loop (one register per
@@ -425,7 +458,7 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
             for (int r = 0; r < NREG; r++)
                 if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) {
                     T* dst = (T*)((char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
-                    if (SK == 1) *dst = acc[ti][tj][r];
+                    if (SK == 1) *dst = LATE_C ? cpre[LATE_C ? ti : 0][LATE_C ? tj : 0][r] + acc[ti][tj][r] : acc[ti][tj][r];
                     else unsafeAtomicAdd(dst, acc[ti][tj][r]);   // hardware global_atomic_add, device scope
                 }
 }

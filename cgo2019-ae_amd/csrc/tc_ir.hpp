@@ -64,6 +64,8 @@ struct Mapping {
     int BXP = 0, BYP = 0, BKP = 0;            // padded to MFMA granularity
     int WX = 1, WY = 1, TX = 1, TY = 1;       // wavefront grid and MFMA tiles per wavefront
     int MI = 0;                               // 0 f64 16x16x4, 1 f32 16x16x4, 2 f32 32x32x2
+    int MINW = 1;                             // resident wavefronts per SIMD asked of the register allocator
+    int LATEC = 0;                            // 1: load the C tile during the first K block instead of before the loop
     int SK = 1;                               // split-K factor: SK workgroups per output tile, atomic accumulate
     int layx = 0, ldx = 0, layy = 0, ldy = 0; // LDS layout per operand
     // model outputs

@@ -63,6 +63,8 @@ std::string Mapping::spec() const
     o << "w=" << WX << "x" << WY << ";t=" << TX << "x" << TY << ";mi=" << MI
       << ";lx=" << layx << ";ly=" << layy;
     if (SK > 1) o << ";sk=" << SK;
+    if (MINW > 1) o << ";mw=" << MINW;
+    if (LATEC) o << ";lc=1";
     return o.str();
 }
 
@@ -198,6 +200,7 @@ bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const 
     if (acc_regs > 256 || acc_regs * 2 > reg_budget) { err = "accumulator tiles exceed the register budget per lane"; return false; }
     if (m.layx < 0 || m.layx > 1 || m.layy < 0 || m.layy > 1) { err = "unknown LDS layout"; return false; }
     if (m.SK < 1 || m.SK > 64) { err = "split-K factor outside 1..64"; return false; }
+    if (m.MINW < 1 || m.MINW > 8 || m.MINW * ceil_div(m.WX * m.WY, arch.simd_per_cu) > 8) { err = "wavefronts per SIMD outside what a block of this size allows"; return false; }
     return true;
 }
 
@@ -510,6 +513,8 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
             if (key == "w") { m.WX = a; m.WY = b; } else { m.TX = a; m.TY = b; }
         } else if (key == "mi") m.MI = atoi(val.c_str());
         else if (key == "sk") m.SK = atoi(val.c_str());
+        else if (key == "mw") m.MINW = atoi(val.c_str());
+        else if (key == "lc") m.LATEC = atoi(val.c_str()) ? 1 : 0;
         else if (key == "lx") lx = atoi(val.c_str());
         else if (key == "ly") ly = atoi(val.c_str());
         else { err = "mapping spec: unknown key " + key; return false; }
@@ -542,7 +547,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6
