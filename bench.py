@@ -157,6 +157,8 @@ def main():
     ap.add_argument("--only-headline", action="store_true", help="skip the table of the other BASELINE configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
     ap.add_argument("--workload", default=HEADLINE, help="expression object to use as the headline workload")
+    ap.add_argument("--suite", default="", help="'tccg': time the 48 TCCG contractions at the sizes of the reference's "
+                    "bench script (cogent/bench_tccg.sh:5-54) and print one JSON line with the table, instead of the headline run")
     ap.add_argument("--copy-only", type=int, default=0, metavar="BYTES",
                     help="only run the plain device-to-device copy kernel on BYTES bytes, --steps times "
                          "(the known-size yardstick the FETCH_SIZE / WRITE_SIZE counter readings are scaled by)")
@@ -180,6 +182,21 @@ def main():
         ms = driver.time_copy(src.data_ptr(), dst.data_ptr(), args.copy_only, args.warmup, args.steps)
         print(json.dumps({"copy_bytes": args.copy_only, "ms_per_copy": ms,
                           "GBps_read_plus_write": round(2 * args.copy_only / ms / 1e6, 1)}))
+        return
+
+    if args.suite:
+        rows = []
+        for e in pkg.manifest():
+            if not e["name"].startswith(args.suite):
+                continue
+            wl = Workload(pkg, tools, e, e["bench_sizes"])
+            r = time_workload(driver, wl, max(1, min(args.warmup, 3)), max(3, min(args.steps, 10)))
+            rows.append(r)
+            print("%-14s %-30s %10.1f us %9.1f GFLOP/s  %s %.3f" % (r["name"], r["sizes"], r["kernel_us_mean"], r["gflops"],
+                                                              r["roofline"]["bound"], r["roofline"]["frac"]), file=sys.stderr, flush=True)
+            del wl
+            torch.cuda.empty_cache()
+        print(json.dumps({"suite": args.suite, "unit": "GFLOP/s", "n_gpus": 1, "data": "synthetic", "rows": rows}))
         return
 
     entry = pkg.manifest_entry(args.workload)

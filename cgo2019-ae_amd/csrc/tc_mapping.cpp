@@ -288,18 +288,21 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     m.blocks_per_cu = r;
     const double waves_simd = (double)(r * W) / arch.simd_per_cu;      // resident wavefronts per SIMD
 
+    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
+    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
     // ---- HBM: a streaming kernel reaches the sustained rate only with about four resident
     // wavefronts per SIMD in different phases (load C / contract / store C); measured 0.75 at two
     const double bw = arch.hbm_bytes_per_s * arch.hbm_sustained_fraction;
     // (wavefronts of one block move in lock-step between barriers, so blocks count too)
     const double occ_eff = std::min(1.0, 0.5 + 0.125 * waves_simd) * (r >= 3 ? 1.0 : r == 2 ? 0.93 : 0.85);
-    m.t_hbm = ((nA + nB) * s + 2.0 * nC * s * c_passes * spread / c_hbm_eff) / (bw * occ_eff);
+    // an input whose tile is shorter than a 64-byte sector along its fastest index is fetched with waste
+    const double nX = m.x_is_a ? nA : nB, nY = m.x_is_a ? nB : nA;
+    auto sector_eff = [&](const std::vector<int>& op) { return std::min(1.0, tile_of(op[0]) * s / 64.0); };
+    m.t_hbm = (nX * s / sector_eff(xop) + nY * s / sector_eff(yop) + 2.0 * nC * s * c_passes * spread / c_hbm_eff) / (bw * occ_eff);
     const double l1_bw = 64.0 * arch.n_cu * arch.clock_hz;
     const double t_l1 = 2.0 * nC * s * c_passes / (l1_bw * c_l1_eff);
 
     // ---- operand slices are re-read by every block that needs them; they mostly hit in L2 / Infinity Cache
-    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
-    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
     auto op_eff = [&](const std::vector<int>& op) {
         double rn = tile_of(op[0]);
         size_t j = 0;
@@ -366,6 +369,13 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
     };
     std::vector<std::vector<int>> x_orders, y_orders, k_orders;
     x_orders.push_back(externals_in(xop, true));          // X must start at C's fastest index
+    {
+        // ... and may continue in the operand's own order, so that the operand's fastest external
+        // index can take a tile even when it is late in C (TCCG-3: C [a,b,c,d], input [d,b,e,a])
+        std::vector<int> o = {c.out_idx[0]};
+        for (int id : xop) if (!c.indices[id].internal && id != c.out_idx[0]) o.push_back(id);
+        if (o != x_orders[0]) x_orders.push_back(o);
+    }
     for (int by_c = 1; by_c >= 0; by_c--) {
         std::vector<int> o = externals_in(yop, by_c != 0);
         if (std::find(y_orders.begin(), y_orders.end(), o) == y_orders.end()) y_orders.push_back(o);
