@@ -1,0 +1,44 @@
+"""The reference's own drivers, unmodified, running against this build (the drop-in demonstration).
+
+oracle/Makefile compiles cogent/drivers/tccg/code_main_tccg_NN.c with its checker switched on
+(-DDEBUG_CORRECTNESS), points the object's call to sd_t_d2_fusion_ at the host-pointer entry
+sd_t_d2_fusion_host_ of lib/tccg_NN_f64.so, and links.  The driver allocates host tensors, fills them
+with rand(), calls the entry point as it would call COGENT's generated code
+(cogent/drivers/tccg/code_main_tccg_01.c:69) and checks the result with ITS host loop and ITS
+tolerance (1e-8 absolute for fp64, 1e-5 for fp32; :135-157).  Skipped where the binaries were not
+built (the reference tree is needed to build them, not to run them).
+"""
+import os
+import re
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CASES = [
+    ("drv_tccg_01", [40, 36, 24, 44]),                 # 3-D output, one contracted index
+    ("drv_tccg_13", [37, 29, 31, 23]),                 # 2-D output, two contracted indices
+    ("drv_tccg_20", [9, 10, 11, 12, 13, 14]),          # 4-D output, two contracted indices
+    ("drv_tccg_31", [12, 8, 6, 12, 8, 6, 12]),         # 6-D output, "-="
+    ("drv_tccg_40", [24, 16, 16, 16, 24, 16, 24]),     # 6-D output at the suite's own extents
+    ("drv_float_tccg_43", [12, 8, 6, 12, 8, 6, 12]),   # fp32
+    ("drv_tccg_01", []),                               # the driver's built-in default extents (16)
+]
+
+
+@pytest.mark.parametrize("binary,sizes", CASES, ids=["%s-%s" % (b, "x".join(map(str, s)) or "default") for b, s in CASES])
+def test_reference_driver_passes_its_own_check(binary, sizes):
+    path = os.path.join(ROOT, "oracle", "_ref", binary)
+    if not os.path.exists(path):
+        pytest.skip("oracle/_ref/%s not built" % binary)
+    print("[gpu] %s %s" % (binary, sizes), flush=True)
+    r = subprocess.run([path] + [str(s) for s in sizes], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout[-2000:]
+    passed = re.search(r"PASSED:\s*([\d,']+)\s+among\s+([\d,']+)", r.stdout)
+    errors = re.search(r"ERROR\s*:\s*([\d,']+)\s+among", r.stdout)
+    assert passed and errors, r.stdout[-2000:]
+    num = lambda s: int(re.sub(r"[,']", "", s))
+    assert num(errors.group(1)) == 0, r.stdout[-2000:]
+    assert num(passed.group(1)) == num(passed.group(2)) > 0
