@@ -66,6 +66,8 @@ struct Mapping {
     int MI = 0;                               // 0 f64 16x16x4, 1 f32 16x16x4, 2 f32 32x32x2
     int MINW = 1;                             // resident wavefronts per SIMD asked of the register allocator
     int LATEC = 0;                            // 1: load the C tile during the first K block instead of before the loop
+    int ntc_forced = -1;                      // -1: decide from the tile shape; 0/1: pinned by a mapping spec (nt=)
+    int NTC = 0;                              // 1: non-temporal C accesses (rows are whole 128-byte lines)
     int SK = 1;                               // split-K factor: SK workgroups per output tile, atomic accumulate
     int layx = 0, ldx = 0, layy = 0, ldy = 0; // LDS layout per operand
     // model outputs

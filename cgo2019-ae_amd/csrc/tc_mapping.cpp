@@ -65,6 +65,7 @@ std::string Mapping::spec() const
     if (SK > 1) o << ";sk=" << SK;
     if (MINW > 1) o << ";mw=" << MINW;
     if (LATEC) o << ";lc=1";
+    if (ntc_forced >= 0) o << ";nt=" << ntc_forced;
     return o.str();
 }
 
@@ -246,6 +247,10 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
         }
     }
     const double seg_bytes = std::min(run, (double)mi.MT) * s;
+    // whole aligned 128-byte lines per lane group: the first X tile is a multiple of a line and the
+    // index's full extent keeps every row start on a line boundary at the representative sizes
+    m.NTC = (m.ntc_forced >= 0) ? m.ntc_forced
+          : (seg_bytes >= 128.0 && ((long long)(m.x_tiles[0] * s) % 128 == 0) && ((long long)(ext(m.x_ids[0]) * s) % 128 == 0)) ? 1 : 0;
     const double c_l1_eff = std::min(1.0, seg_bytes / 128.0);
     // contiguous chunk of C owned by one block (bytes): whole 128-byte lines or not
     double chunk = 1;
@@ -525,6 +530,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "sk") m.SK = atoi(val.c_str());
         else if (key == "mw") m.MINW = atoi(val.c_str());
         else if (key == "lc") m.LATEC = atoi(val.c_str()) ? 1 : 0;
+        else if (key == "nt") m.ntc_forced = atoi(val.c_str()) ? 1 : 0;
         else if (key == "lx") lx = atoi(val.c_str());
         else if (key == "ly") ly = atoi(val.c_str());
         else { err = "mapping spec: unknown key " + key; return false; }
@@ -557,7 +563,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6
