@@ -175,34 +175,39 @@ __device__ __forceinline__ void slice_store(const typename Cfg::T (&reg)[SLOTS],
     }
 }
 
-// Element offsets, relative to the block's C tile origin, of the accumulator elements a lane holds:
-// cx[tj] for its column in MFMA tile column tj, cy[ti][r] for the row of register r in tile row ti;
+// Element offsets, relative to the block's C tile origin, of the accumulator elements a lane holds.
+// Normal roles (X along MFMA columns): cx[tj][0] for the lane's column in tile column tj, cy[ti][r] for
+// the row of register r in tile row ti.  Swapped roles (SWP, X along MFMA rows): cx[tj][r], cy[ti][0].
 // -1 marks positions outside the tensor (ragged tiles, padding).
-template <class Cfg, bool EXT_FULL>
+template <class Cfg, bool EXT_FULL, bool SWP>
 __device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const int* rem, const TcDims& d,
-                                               int (&cx)[Cfg::TX], int (&cy)[Cfg::TY][Mfma<Cfg::MI>::NREG])
+                                               int (&cx)[Cfg::TX][SWP ? Mfma<Cfg::MI>::NREG : 1],
+                                               int (&cy)[Cfg::TY][SWP ? 1 : Mfma<Cfg::MI>::NREG])
 {
     typedef Mfma<Cfg::MI> MM;
     constexpr int MT = MM::MT, NREG = MM::NREG, TX = Cfg::TX, TY = Cfg::TY;
 #pragma unroll
     for (int tj = 0; tj < TX; tj++) {
-        const int x = (wx * TX + tj) * MT + lane % MT;
-        unsigned q = (unsigned)x;
-        int off = 0; bool ok = (Cfg::BXP == Cfg::BX) || (x < Cfg::BX);
 #pragma unroll
-        for (int i = 0; i < Cfg::NX; i++) {
-            const int c = (int)(q % (unsigned)Cfg::x_tile(i));
-            q /= (unsigned)Cfg::x_tile(i);
-            off += c * d.sC[Cfg::x_id(i)];
-            if (!EXT_FULL) ok = ok && (c < rem[Cfg::x_id(i)]);
+        for (int r = 0; r < (SWP ? NREG : 1); r++) {
+            const int x = (wx * TX + tj) * MT + (SWP ? MM::row(r, lane) : lane % MT);
+            unsigned q = (unsigned)x;
+            int off = 0; bool ok = (Cfg::BXP == Cfg::BX) || (x < Cfg::BX);
+#pragma unroll
+            for (int i = 0; i < Cfg::NX; i++) {
+                const int c = (int)(q % (unsigned)Cfg::x_tile(i));
+                q /= (unsigned)Cfg::x_tile(i);
+                off += c * d.sC[Cfg::x_id(i)];
+                if (!EXT_FULL) ok = ok && (c < rem[Cfg::x_id(i)]);
+            }
+            cx[tj][r] = ok ? off : -1;
         }
-        cx[tj] = ok ? off : -1;
     }
 #pragma unroll
     for (int ti = 0; ti < TY; ti++) {
 #pragma unroll
-        for (int r = 0; r < NREG; r++) {
-            const int y = (wy * TY + ti) * MT + MM::row(r, lane);
+        for (int r = 0; r < (SWP ? 1 : NREG); r++) {
+            const int y = (wy * TY + ti) * MT + (SWP ? lane % MT : MM::row(r, lane));
             unsigned q = (unsigned)y;
             int off = 0; bool ok = (Cfg::BYP == Cfg::BY) || (y < Cfg::BY);
 #pragma unroll
@@ -225,7 +230,28 @@ __device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const i
 // ONE_KB: the whole contracted range fits one K block (every contracted extent <= its tile), the
 // shape of the HBM-bound many-index contractions.  The K loop, its odometer and the register
 // prefetch of the next slices disappear, which frees registers for more resident wavefronts.
-template <class Cfg, bool EXT_FULL, bool INT_FULL, bool ONE_KB>
+//
+// SWP (fp32 only): the X side runs along the MFMA ROWS instead of the columns.  In the fp32 MFMA
+// layouts a lane holds 4 consecutive rows per register group, so with C's fastest index on the rows
+// each lane owns 16 contiguous bytes of C and the tile is read and written with one 128-bit access
+// per group -- a wavefront covers a contiguous kilobyte per instruction where the column layout
+// gives 64-byte pieces.  The launcher uses it when the fastest extent is a multiple of 4 and C is
+// 16-byte aligned.
+// f(integral_constant<int, 0>), .., f(integral_constant<int, N - 1>), unconditionally
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) { f(std::integral_constant<int, I>()); static_for<N, I + 1>(f); }
+}
+// f(0), f(1), .. while the index is below both N and n: every call sits inside the branch of the one
+// before it, so control reaches call I only from call I - 1
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_chain(int n, F&& f)
+{
+    if constexpr (I < N) { if (I < n) { f(std::integral_constant<int, I>()); static_chain<N, I + 1>(n, f); } }
+}
+
+template <class Cfg, bool EXT_FULL, bool INT_FULL, bool ONE_KB, bool SWP>
 __global__ __launch_bounds__(Cfg::NT, Cfg::MINW)     // MINW: wavefronts per SIMD the register allocator must leave room for
 void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __restrict__ X,
                     const typename Cfg::T* __restrict__ Y, const TcDims d)
@@ -312,9 +338,16 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     const T* __restrict__ Yb = Y + uniform64(baseY);
 
     // ---- where this lane's accumulator elements live in C (-1: outside)
-    int cx[TX];
-    int cy[TY][NREG];
-    c_tile_offsets<Cfg, EXT_FULL>(lane, wx, wy, rem, d, cx, cy);
+    int cx[TX][SWP ? NREG : 1];
+    int cy[TY][SWP ? 1 : NREG];
+    c_tile_offsets<Cfg, EXT_FULL, SWP>(lane, wx, wy, rem, d, cx, cy);
+    // offset of accumulator element (ti, tj, r) and whether it is inside the tensor
+    auto c_off = [&](int ti, int tj, int r) -> int { return cx[tj][SWP ? r : 0] + cy[ti][SWP ? 0 : r]; };
+    auto c_ok = [&](int ti, int tj, int r) -> bool {
+        return (EXT_FULL && !PADDED) || (cx[tj][SWP ? r : 0] >= 0 && cy[ti][SWP ? 0 : r] >= 0);
+    };
+    typedef T T4 __attribute__((ext_vector_type(4)));
+    constexpr bool VEC4 = SWP;      // 4 consecutive registers = 4 consecutive elements of C's fastest index
 
     // ---- accumulators start from the C tile: C_in + sum, summed in k order.
     // LATE_C: they start from zero instead and the C tile is loaded into registers of its own during
@@ -327,13 +360,26 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
     for (int ti = 0; ti < TY; ti++)
 #pragma unroll
-        for (int tj = 0; tj < TX; tj++)
+        for (int tj = 0; tj < TX; tj++) {
+            if (VEC4) {
 #pragma unroll
-            for (int r = 0; r < NREG; r++) {
-                T v = (T)0;
-                if (SK == 1 && !LATE_C && ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0))) v = c_load<Cfg::NTC != 0>((const T*)((const char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T)));
-                acc[ti][tj][r] = v;
+                for (int g = 0; g < NREG / 4; g++) {
+                    T4 v = {(T)0, (T)0, (T)0, (T)0};
+                    if (SK == 1 && !LATE_C && c_ok(ti, tj, 4 * g))
+                        v = c_load<(Cfg::NTC & 1) != 0>((const T4*)((const char*)Cb + (unsigned)c_off(ti, tj, 4 * g) * (unsigned)sizeof(T)));
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[ti][tj][4 * g + e] = v[e];
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < NREG; r++) {
+                    T v = (T)0;
+                    if (SK == 1 && !LATE_C && c_ok(ti, tj, r))
+                        v = c_load<(Cfg::NTC & 1) != 0>((const T*)((const char*)Cb + (unsigned)c_off(ti, tj, r) * (unsigned)sizeof(T)));
+                    acc[ti][tj][r] = v;
+                }
             }
+        }
 
     // ---- padding rows/columns of the LDS slices are never written by the staging: clear once
     if (PADDED) {
@@ -366,9 +412,42 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         }
     }
 
-    T rx[SLOTS_X], ry[SLOTS_Y];
-    slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb + uniform64(kx0), d, rem, tid);
-    slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb + uniform64(ky0), d, rem, tid);
+    // Prefetch depth PD: the slices of K block kb + PD are requested while block kb is contracted,
+    // each depth in registers of its own (stage kb % PD, a compile-time index in every copy of the
+    // trip below).  One trip of MFMA work is a fraction of a microsecond; a slice gathered through a
+    // busy L2 takes several times that, so one stage of look-ahead leaves the loop waiting on loads.
+    constexpr int PD = ONE_KB ? 1 : Cfg::PD;
+    T rx[PD][SLOTS_X], ry[PD][SLOTS_Y];
+    int64_t kxh = kx0, kyh = ky0;                  // slice origin of the newest K block requested
+    int head = 0;                                  // ... and its number within this workgroup's share
+    // Move the head one K block on (first composite K index fastest) -- unless it is at the last one:
+    // then the same block is requested again and never used.  Every trip thus issues the same loads
+    // whatever the trip count, which keeps the outstanding-load count known at compile time: the wait
+    // before a stage is stored to LDS then leaves the PD - 1 newer stages in flight.
+    auto advance_head = [&]() {
+        if (head + 1 < nkb) {
+            head++;
+            kxh = 0; kyh = 0;
+            bool carry = true;
+#pragma unroll
+            for (int i = 0; i < Cfg::NK; i++) {
+                const int id = Cfg::k_id(i);
+                if (carry) { kbc[i]++; carry = false; if (kbc[i] == d.nblk[id]) { kbc[i] = 0; carry = true; } }
+                const int o = kbc[i] * Cfg::k_tile(i);
+                rem[id] = d.ext[id] - o;
+                kxh += (int64_t)o * d.sX[id];
+                kyh += (int64_t)o * d.sY[id];
+            }
+        }
+    };
+    slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx[0], Xb + uniform64(kxh), d, rem, tid);
+    slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry[0], Yb + uniform64(kyh), d, rem, tid);
+#pragma unroll
+    for (int s = 1; s < PD; s++) {
+        advance_head();
+        slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx[s], Xb + uniform64(kxh), d, rem, tid);
+        slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry[s], Yb + uniform64(kyh), d, rem, tid);
+    }
 
     if (!ONE_KB) {
         // Drain the C-tile and first-slice loads BEFORE the K loop.  Otherwise the compiler has to
@@ -378,36 +457,30 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         __builtin_amdgcn_s_waitcnt(0x0F70);
     }
     if (NBUF == 2) {
-        slice_store<Cfg, OX, false>(rx, lds_x_all, d, tid);
-        slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y_all, d, tid);
+        slice_store<Cfg, OX, false>(rx[0], lds_x_all, d, tid);
+        slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry[0], lds_y_all, d, tid);
         __syncthreads();
     }
-    auto k_block = [&](const int kb, auto first_trip) {
+    // One trip: contract K block kb, whose slices are (NBUF == 2) already in LDS or (NBUF == 1) in
+    // stage S = kb % PD.
+    auto k_block = [&](const int kb, auto stage, auto first_trip) {
+        constexpr int S = decltype(stage)::value, SN = (S + 1) % PD;
         T* lds_x = lds_x_all + (NBUF == 2 ? (kb & 1) * LDS_X : 0);
         T* lds_y = lds_y_all + (NBUF == 2 ? (kb & 1) * LDS_Y : 0);
         if (NBUF == 1) {
             if (!ONE_KB) __syncthreads();      // previous slices fully consumed
-            slice_store<Cfg, OX, false>(rx, lds_x, d, tid);
-            slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y, d, tid);
+            slice_store<Cfg, OX, false>(rx[S], lds_x, d, tid);
+            slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry[S], lds_y, d, tid);
             __syncthreads();
         }
 
-        const bool more = !ONE_KB && (kb + 1 < nkb);
-        if (more) {
-            // advance the K-block odometer (first composite K index fastest) and prefetch
-            int64_t kx = 0, ky = 0;
-            bool carry = true;
-#pragma unroll
-            for (int i = 0; i < Cfg::NK; i++) {
-                const int id = Cfg::k_id(i);
-                if (carry) { kbc[i]++; carry = false; if (kbc[i] == d.nblk[id]) { kbc[i] = 0; carry = true; } }
-                const int o = kbc[i] * Cfg::k_tile(i);
-                rem[id] = d.ext[id] - o;
-                kx += (int64_t)o * d.sX[id];
-                ky += (int64_t)o * d.sY[id];
-            }
-            slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx, Xb + uniform64(kx), d, rem, tid);
-            slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry, Yb + uniform64(ky), d, rem, tid);
+        // with one stage nothing newer is in flight, so the last trip can simply skip the request
+        const bool more = PD > 1 || kb + 1 < nkb;
+        if (!ONE_KB && more) {
+            // stage S is free (its slices are in LDS): request K block kb + PD into it
+            advance_head();
+            slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx[S], Xb + uniform64(kxh), d, rem, tid);
+            slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry[S], Yb + uniform64(kyh), d, rem, tid);
         }
         if (LATE_C && decltype(first_trip)::value) {
 #pragma unroll
@@ -417,8 +490,8 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
                     for (int r = 0; r < NREG; r++) {
                         T v = (T)0;
-                        if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0))
-                            v = c_load<Cfg::NTC != 0>((const T*)((const char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T)));
+                        if (c_ok(ti, tj, r))
+                            v = c_load<(Cfg::NTC & 1) != 0>((const T*)((const char*)Cb + (unsigned)c_off(ti, tj, r) * (unsigned)sizeof(T)));
                         cpre[LATE_C ? ti : 0][LATE_C ? tj : 0][r] = v;
                     }
         }
@@ -434,20 +507,30 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
             for (int ti = 0; ti < TY; ti++)
 #pragma unroll
-                for (int tj = 0; tj < TX; tj++) acc[ti][tj] = MM::mma(a[ti], b[tj], acc[ti][tj]);
+                for (int tj = 0; tj < TX; tj++) acc[ti][tj] = SWP ? MM::mma(b[tj], a[ti], acc[ti][tj]) : MM::mma(a[ti], b[tj], acc[ti][tj]);
         }
 
         if (NBUF == 2) {
+            // the slices of K block kb + 1 go to the other LDS buffer (after the last block: the
+            // unused repeat of it, harmless)
             if (more) {
-                slice_store<Cfg, OX, false>(rx, lds_x_all + ((kb + 1) & 1) * LDS_X, d, tid);
-                slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry, lds_y_all + ((kb + 1) & 1) * LDS_Y, d, tid);
+                slice_store<Cfg, OX, false>(rx[SN], lds_x_all + ((kb + 1) & 1) * LDS_X, d, tid);
+                slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry[SN], lds_y_all + ((kb + 1) & 1) * LDS_Y, d, tid);
             }
             __syncthreads();
         }
     };
-    // the first trip is a copy of its own so that what is in flight during it is known exactly
-    k_block(0, std::true_type());
-    for (int kb = 1; kb < nkb; kb++) k_block(kb, std::false_type());
+    // The first trip is a copy of its own so that what is in flight during it is known exactly; then
+    // whole groups of PD trips (stage indices 1, 2, .., 0), then the at most PD - 1 trips left over,
+    // each entered only from the one before it so that no two load histories meet.
+    k_block(0, std::integral_constant<int, 0>(), std::true_type());
+    if (!ONE_KB) {
+        int kb = 1;
+        for (; kb + PD <= nkb; kb += PD)
+            static_for<PD>([&](auto s) { k_block(kb + decltype(s)::value, std::integral_constant<int, (1 + decltype(s)::value) % PD>(), std::false_type()); });
+        const int left = nkb - kb;
+        static_chain<PD - 1>(left, [&](auto s) { k_block(kb + decltype(s)::value, std::integral_constant<int, (1 + decltype(s)::value) % PD>(), std::false_type()); });
+    }
 
     // ---- write the tile back.  With a K loop the offsets are derived again here from an opaque
     // copy of the lane id instead of being kept in registers across the loop (one register per
@@ -455,19 +538,32 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     if (!ONE_KB) {
         int lane2 = lane;
         asm volatile("" : "+v"(lane2));
-        c_tile_offsets<Cfg, EXT_FULL>(lane2, wx, wy, rem, d, cx, cy);
+        c_tile_offsets<Cfg, EXT_FULL, SWP>(lane2, wx, wy, rem, d, cx, cy);
     }
 #pragma unroll
     for (int ti = 0; ti < TY; ti++)
 #pragma unroll
-        for (int tj = 0; tj < TX; tj++)
+        for (int tj = 0; tj < TX; tj++) {
+            if (VEC4 && SK == 1) {
 #pragma unroll
-            for (int r = 0; r < NREG; r++)
-                if ((EXT_FULL && !PADDED) || (cx[tj] >= 0 && cy[ti][r] >= 0)) {
-                    T* dst = (T*)((char*)Cb + (unsigned)(cx[tj] + cy[ti][r]) * (unsigned)sizeof(T));
-                    if (SK == 1) c_store<Cfg::NTC != 0>(LATE_C ? cpre[LATE_C ? ti : 0][LATE_C ? tj : 0][r] + acc[ti][tj][r] : acc[ti][tj][r], dst);
-                    else unsafeAtomicAdd(dst, acc[ti][tj][r]);   // hardware global_atomic_add, device scope
-                }
+                for (int g = 0; g < NREG / 4; g++)
+                    if (c_ok(ti, tj, 4 * g)) {
+                        T4 v;
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            v[e] = LATE_C ? cpre[LATE_C ? ti : 0][LATE_C ? tj : 0][4 * g + e] + acc[ti][tj][4 * g + e] : acc[ti][tj][4 * g + e];
+                        c_store<(Cfg::NTC & 2) != 0>(v, (T4*)((char*)Cb + (unsigned)c_off(ti, tj, 4 * g) * (unsigned)sizeof(T)));
+                    }
+            } else {
+#pragma unroll
+                for (int r = 0; r < NREG; r++)
+                    if (c_ok(ti, tj, r)) {
+                        T* dst = (T*)((char*)Cb + (unsigned)c_off(ti, tj, r) * (unsigned)sizeof(T));
+                        if (SK == 1) c_store<(Cfg::NTC & 2) != 0>(LATE_C ? cpre[LATE_C ? ti : 0][LATE_C ? tj : 0][r] + acc[ti][tj][r] : acc[ti][tj][r], dst);
+                        else unsafeAtomicAdd(dst, acc[ti][tj][r]);   // hardware global_atomic_add, device scope
+                    }
+            }
+        }
 }
 
 // ---------------------------------------------------------------------------

@@ -44,6 +44,31 @@ inline int tc_check_launch(const char* what)
 
 enum TcVariant { TC_VARIANT_AUTO = 0, TC_VARIANT_PLAIN = 1, TC_VARIANT_TILED = 2 };
 
+template <class Cfg, bool ONE_KB, bool SWP>
+inline void tc_launch_full_partial(bool ext_full, bool int_full, dim3 g, dim3 b, hipStream_t stream,
+                                   typename Cfg::T* c, const typename Cfg::T* x, const typename Cfg::T* y, const TcDims& d)
+{
+    if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, ONE_KB, SWP>),   g, b, 0, stream, c, x, y, d);
+    else if (ext_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false, ONE_KB, SWP>),  g, b, 0, stream, c, x, y, d);
+    else if (int_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true, ONE_KB, SWP>),  g, b, 0, stream, c, x, y, d);
+    else                        hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false, ONE_KB, SWP>), g, b, 0, stream, c, x, y, d);
+}
+
+template <class Cfg>
+inline void tc_launch_variant(bool one_kb, bool ext_full, bool int_full, bool swp, dim3 g, dim3 b, hipStream_t stream,
+                              typename Cfg::T* c, const typename Cfg::T* x, const typename Cfg::T* y, const TcDims& d)
+{
+    if constexpr (Cfg::SWAP != 0) {
+        if (swp) {
+            if (one_kb) tc_launch_full_partial<Cfg, true, true>(ext_full, int_full, g, b, stream, c, x, y, d);
+            else        tc_launch_full_partial<Cfg, false, true>(ext_full, int_full, g, b, stream, c, x, y, d);
+            return;
+        }
+    }
+    if (one_kb) tc_launch_full_partial<Cfg, true, false>(ext_full, int_full, g, b, stream, c, x, y, d);
+    else        tc_launch_full_partial<Cfg, false, false>(ext_full, int_full, g, b, stream, c, x, y, d);
+}
+
 // sizes[] holds one extent per index id: output indices in output order, then
 // the contracted indices in sum() order -- the order of the entry point's
 // `int size_*` parameters (cogent/src/codes/kernels/tc_interface.py:1459-1492).
@@ -136,17 +161,9 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     const T* y = (const T*)(Cfg::X_IS_A ? B : A);
     const dim3 g((unsigned)grid), b(Cfg::NT);
     tc_clear_hip_error();
-    if (nkb == 1) {
-        if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, true>),    g, b, 0, stream, c, x, y, d);
-        else if (ext_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false, true>),   g, b, 0, stream, c, x, y, d);
-        else if (int_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true, true>),   g, b, 0, stream, c, x, y, d);
-        else                        hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false, true>),  g, b, 0, stream, c, x, y, d);
-    } else {
-        if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, false>),   g, b, 0, stream, c, x, y, d);
-        else if (ext_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false, false>),  g, b, 0, stream, c, x, y, d);
-        else if (int_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true, false>),  g, b, 0, stream, c, x, y, d);
-        else                        hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false, false>), g, b, 0, stream, c, x, y, d);
-    }
+    // swapped MFMA roles with 128-bit C accesses: fp32 only, fastest extent a multiple of 4, C 16-byte aligned
+    const bool swp = Cfg::SWAP && (sizes[Cfg::c_id(0)] % 4 == 0) && (((uintptr_t)C & 15) == 0);
+    tc_launch_variant<Cfg>(nkb == 1, ext_full, int_full, swp, g, b, stream, c, x, y, d);
     return tc_check_launch("tiled kernel launch failed");
 }
 

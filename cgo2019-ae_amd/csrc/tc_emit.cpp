@@ -91,7 +91,7 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
     operand("X", xop, m.x_ids, m.x_tiles);
     operand("Y", yop, m.y_ids, m.y_tiles);
     o << "    static constexpr int WX = " << m.WX << ", WY = " << m.WY << ", TX = " << m.TX << ", TY = " << m.TY << ", NT = " << 64 * m.WX * m.WY << ";\n";
-    o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ";\n";
+    o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ";\n";
     o << "    static constexpr int LAYX = " << m.layx << ", LDX = " << m.ldx << ", LAYY = " << m.layy << ", LDY = " << m.ldy << ";\n";
     o << "};\n";
     o << "}  // namespace\n\n";

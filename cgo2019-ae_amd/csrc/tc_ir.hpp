@@ -66,8 +66,12 @@ struct Mapping {
     int MI = 0;                               // 0 f64 16x16x4, 1 f32 16x16x4, 2 f32 32x32x2
     int MINW = 1;                             // resident wavefronts per SIMD asked of the register allocator
     int LATEC = 0;                            // 1: load the C tile during the first K block instead of before the loop
-    int ntc_forced = -1;                      // -1: decide from the tile shape; 0/1: pinned by a mapping spec (nt=)
-    int NTC = 0;                              // 1: non-temporal C accesses (rows are whole 128-byte lines)
+    int ntc_forced = -1;                      // -1: decide from the tile shape; 0..3: pinned by a mapping spec (nt=)
+    int NTC = 0;                              // non-temporal C accesses: bit 0 loads, bit 1 stores (both when rows are whole 128-byte lines)
+    int SWAP = 0;                             // 1 (fp32): C's fastest index on the MFMA rows, 128-bit C accesses
+    int swap_forced = -1;
+    int PD = 1;                               // K blocks requested ahead of the one being contracted (register stages)
+    int pd_forced = -1;
     int SK = 1;                               // split-K factor: SK workgroups per output tile, atomic accumulate
     int layx = 0, ldx = 0, layy = 0, ldy = 0; // LDS layout per operand
     // model outputs

@@ -66,6 +66,8 @@ std::string Mapping::spec() const
     if (MINW > 1) o << ";mw=" << MINW;
     if (LATEC) o << ";lc=1";
     if (ntc_forced >= 0) o << ";nt=" << ntc_forced;
+    if (swap_forced >= 0) o << ";sw=" << swap_forced;
+    if (pd_forced >= 1) o << ";pd=" << pd_forced;
     return o.str();
 }
 
@@ -162,7 +164,9 @@ static void finish_geometry(const Contraction& c, DType t, Mapping& m)
     const int ex = m.layx == 0 ? m.BKP * m.ldx : m.BXP * m.ldx;
     const int ey = m.layy == 0 ? m.BKP * m.ldy : m.BYP * m.ldy;
     m.lds_bytes = (ex + ey) * esize(t);
-    (void)c;
+    // fp32: put C's fastest index on the MFMA rows when its tile is a multiple of 4 (128-bit C accesses)
+    const bool can_swap = t == DType::F32 && !m.x_tiles.empty() && m.x_ids[0] == c.out_idx[0] && m.x_tiles[0] % 4 == 0;
+    m.SWAP = can_swap && (m.swap_forced != 0) ? 1 : 0;
 }
 
 bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const Mapping& m, std::string& err)
@@ -250,7 +254,7 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     // whole aligned 128-byte lines per lane group: the first X tile is a multiple of a line and the
     // index's full extent keeps every row start on a line boundary at the representative sizes
     m.NTC = (m.ntc_forced >= 0) ? m.ntc_forced
-          : (seg_bytes >= 128.0 && ((long long)(m.x_tiles[0] * s) % 128 == 0) && ((long long)(ext(m.x_ids[0]) * s) % 128 == 0)) ? 1 : 0;
+          : (seg_bytes >= 128.0 && ((long long)(m.x_tiles[0] * s) % 128 == 0) && ((long long)(ext(m.x_ids[0]) * s) % 128 == 0)) ? 3 : 0;
     const double c_l1_eff = std::min(1.0, seg_bytes / 128.0);
     // contiguous chunk of C owned by one block (bytes): whole 128-byte lines or not
     double chunk = 1;
@@ -281,6 +285,12 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const int slots = (int)(std::ceil((double)m.BK * m.BX / (64.0 * W)) + std::ceil((double)m.BK * m.BY / (64.0 * W)));
     int regs = acc_regs + 40 + slots * r4 + (m.TX + m.TY * mi.NREG) + (m.TX + m.TY) * r4;
     if (nkb > 1) regs += 2 * slots;
+    // prefetch depth: one K block ahead unless a mapping spec asks for more (pd=); each extra stage
+    // holds one slice share in registers, and on the shapes measured so far the registers were worth
+    // more as a resident wavefront
+    m.PD = 1;
+    if (nkb > 1 && m.pd_forced >= 1) m.PD = m.pd_forced;
+    regs += (m.PD - 1) * slots * (r4 + 1);
     const int reg_cap = std::min(512, arch.vgpr_per_lane / ceil_div(W, arch.simd_per_cu));
     const double spill_penalty = regs > reg_cap ? 1.0 + 2.0 * (double)(regs - reg_cap) / reg_cap : 1.0;
     int waves_per_simd = std::max(1, std::min(8, arch.vgpr_per_lane / std::max(regs, 64)));
@@ -530,7 +540,9 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "sk") m.SK = atoi(val.c_str());
         else if (key == "mw") m.MINW = atoi(val.c_str());
         else if (key == "lc") m.LATEC = atoi(val.c_str()) ? 1 : 0;
-        else if (key == "nt") m.ntc_forced = atoi(val.c_str()) ? 1 : 0;
+        else if (key == "nt") m.ntc_forced = std::max(0, std::min(3, atoi(val.c_str())));
+        else if (key == "sw") m.swap_forced = atoi(val.c_str()) ? 1 : 0;
+        else if (key == "pd") m.pd_forced = std::max(1, std::min(8, atoi(val.c_str())));
         else if (key == "lx") lx = atoi(val.c_str());
         else if (key == "ly") ly = atoi(val.c_str());
         else { err = "mapping spec: unknown key " + key; return false; }
@@ -563,7 +575,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

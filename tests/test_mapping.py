@@ -40,11 +40,11 @@ def check_mapping(info, m, dtype):
     blocks = 1
     for name, t in m["x"] + m["y"]:
         blocks *= -(-ext[name] // t)
-    assert m["model"]["blocks"] == blocks
+    assert m["model"]["blocks"] == blocks * m["split_k"]         # split K: that many workgroups per output tile
     ksteps = 1
     for name, t in m["k"]:
         ksteps *= -(-ext[name] // t)
-    assert m["model"]["k_steps"] == ksteps
+    assert m["model"]["k_steps"] == -(-ksteps // m["split_k"])    # K blocks per workgroup
     assert m["model"]["cost_us"] > 0
 
 
@@ -76,6 +76,33 @@ def test_manual_rank_and_spec_round_trip(tools):
     assert same.info["mapping"] == third.info["mapping"]
     named = tools.plan(text, "DOUBLE", mapping_spec="x=d:24,c:4;y=b:24,a:4;k=e:8;w=2x2;t=3x3")
     assert named.info["mapping"]["block_tile"] == [96, 96, 8] and named.info["mapping"]["threads"] == 256
+
+
+def test_kernel_options_in_a_spec(tools):
+    """pd= (K blocks requested ahead), nt= (non-temporal C: bit 0 loads, bit 1 stores), sw= (fp32: C's fastest
+    index on the MFMA rows), lc=, mw=, sk= are carried into the plan and back out through its spec."""
+    text = open(os.path.join(EXPR_DIR, "cfg2_f64.in")).read()
+    base = "x=d:24,c:4;y=b:24,a:4;k=e:8;w=2x2;t=3x3"
+    m = tools.plan(text, "DOUBLE", mapping_spec=base).info["mapping"]
+    assert m["prefetch_depth"] == 1 and m["swapped_roles"] == 0 and m["nontemporal_c"] == 0   # 192-byte rows
+    m = tools.plan(text, "DOUBLE", mapping_spec=base + ";pd=3;nt=2;mw=2;lc=1").info["mapping"]
+    assert m["prefetch_depth"] == 3 and m["nontemporal_c"] == 2 and m["min_waves_per_simd"] == 2 and m["late_c"] == 1
+    assert "pd=3" in m["spec"] and "nt=2" in m["spec"]
+    again = tools.plan(text, "DOUBLE", mapping_spec=m["spec"]).info["mapping"]
+    assert again == m
+    # fp32 with a fastest tile that is a multiple of 4: swapped roles by default, sw=0 turns them off
+    text4 = open(os.path.join(EXPR_DIR, "cfg4_16_f32.in")).read()
+    auto = tools.plan(text4, "FLOAT").info["mapping"]
+    assert auto["swapped_roles"] == 1 and auto["nontemporal_c"] == 0           # 64-byte rows: no whole lines per access
+    off = tools.plan(text4, "FLOAT", mapping_spec=auto["spec"] + ";sw=0").info["mapping"]
+    assert off["swapped_roles"] == 0
+    # fp64 rows of 16 elements are whole aligned lines: non-temporal loads and stores
+    text5 = open(os.path.join(EXPR_DIR, "cfg5_1_f64.in")).read()
+    assert tools.plan(text5, "DOUBLE").info["mapping"]["nontemporal_c"] == 3
+    # a fastest tile that is not a multiple of 4 cannot use 128-bit accesses
+    odd = tools.plan("t3 [a,30,b,64] += sum(c,64) * t2 [a,c] * v2 [c,b];", "FLOAT",
+                     mapping_spec="x=a:30;y=b:32;k=c:8;w=1x1;t=2x2;mi=1").info["mapping"]
+    assert odd["swapped_roles"] == 0
 
 
 BAD_SPECS = [
