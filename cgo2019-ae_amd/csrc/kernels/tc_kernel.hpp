@@ -567,6 +567,33 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 }
 
 // ---------------------------------------------------------------------------
+// Repack kernel: out = the input with its indices permuted, dense, ext[]/sin[]
+// listed in the OUTPUT order (fastest first).  One lane per element, writes
+// coalesced; the reads are a gather, which is fine for the inputs this is used
+// on: a few megabytes next to an output of hundreds, mostly served from L2.
+struct TcRepackDims {
+    int n;
+    int ext[TC_MAXI], sin[TC_MAXI];
+    long long total;
+};
+
+template <class T>
+__global__ __launch_bounds__(256)
+void tc_repack_kernel(const T* __restrict__ in, T* __restrict__ out, const TcRepackDims p)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= p.total) return;
+    unsigned q = (unsigned)i;
+    unsigned off = 0;
+    for (int j = 0; j < p.n; j++) {
+        const unsigned e = (unsigned)p.ext[j];
+        off += (q % e) * (unsigned)p.sin[j];
+        q /= e;
+    }
+    out[i] = in[off];
+}
+
+// ---------------------------------------------------------------------------
 // Plain kernel: one lane per output element, contracted indices walked in
 // sum() order with separately rounded multiply and add, i.e. the summation
 // order of the reference's host check (cogent/drivers/tccg/code_main_tccg_01.c:117-133).

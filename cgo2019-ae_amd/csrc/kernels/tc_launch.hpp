@@ -22,7 +22,7 @@ enum TcStatus {
     TC_ERR_TOO_LARGE = 3,      // a tensor has 2^31 or more elements, or the grid does not fit
     TC_ERR_LAUNCH = 4,         // the HIP runtime refused the launch
     TC_ERR_BAD_VARIANT = 5,
-    TC_ERR_ALLOC = 6,          // host-pointer shim only
+    TC_ERR_ALLOC = 6,          // host-pointer shim, or the stream-ordered buffer of a repacked input
 };
 
 inline char* tc_error_buffer() { static thread_local char buf[256] = ""; return buf; }
@@ -121,8 +121,11 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
 
     TcDims d;
     memset(&d, 0, sizeof(d));
-    const int64_t* sX = Cfg::X_IS_A ? sA : sB;
-    const int64_t* sY = Cfg::X_IS_A ? sB : sA;
+    // strides of the two inputs as the kernel reads them: the tensors' own, or dense in tile order
+    // for an input that is repacked below
+    int64_t sX[TC_MAXI] = {0}, sY[TC_MAXI] = {0};
+    { int64_t n = 1; for (int j = 0; j < Cfg::XR; j++) { sX[Cfg::xo_id(j)] = n; n *= sizes[Cfg::xo_id(j)]; } }
+    { int64_t n = 1; for (int j = 0; j < Cfg::YR; j++) { sY[Cfg::yo_id(j)] = n; n *= sizes[Cfg::yo_id(j)]; } }
     for (int i = 0; i < Cfg::NIDX; i++) {
         d.ext[i] = sizes[i]; d.nblk[i] = 1;
         d.sC[i] = (int)sC[i]; d.sX[i] = (int)sX[i]; d.sY[i] = (int)sY[i];
@@ -159,12 +162,47 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     T* c = (T*)C;
     const T* x = (const T*)(Cfg::X_IS_A ? A : B);
     const T* y = (const T*)(Cfg::X_IS_A ? B : A);
-    const dim3 g((unsigned)grid), b(Cfg::NT);
     tc_clear_hip_error();
+
+    // Repacked inputs: a copy in tile order (tiled externals, then K), made on the same stream in
+    // memory that is allocated and freed in stream order, so calls on different streams do not share it.
+    T* ws = nullptr;
+    if (Cfg::RPX || Cfg::RPY) {
+        const int64_t nx = Cfg::X_IS_A ? nA : nB, ny = Cfg::X_IS_A ? nB : nA;
+        const int64_t off_y = Cfg::RPX ? ((nx + 31) / 32) * 32 : 0;              // keep the second copy 256-byte aligned
+        const int64_t total = off_y + (Cfg::RPY ? ny : 0);
+        if (hipMallocAsync((void**)&ws, (size_t)total * sizeof(T), stream) != hipSuccess || !ws) {
+            (void)hipGetLastError();
+            return tc_fail(TC_ERR_ALLOC, "stream-ordered allocation of the repack buffer failed");
+        }
+        const int64_t* sXin = Cfg::X_IS_A ? sA : sB;
+        const int64_t* sYin = Cfg::X_IS_A ? sB : sA;
+        if (Cfg::RPX) {
+            TcRepackDims r;
+            memset(&r, 0, sizeof(r));
+            r.n = Cfg::XR; r.total = nx;
+            for (int j = 0; j < Cfg::XR; j++) { r.ext[j] = sizes[Cfg::xo_id(j)]; r.sin[j] = (int)sXin[Cfg::xo_id(j)]; }
+            hipLaunchKernelGGL(tc_repack_kernel<T>, dim3((unsigned)((nx + 255) / 256)), dim3(256), 0, stream, x, ws, r);
+            x = ws;
+        }
+        if (Cfg::RPY) {
+            TcRepackDims r;
+            memset(&r, 0, sizeof(r));
+            r.n = Cfg::YR; r.total = ny;
+            for (int j = 0; j < Cfg::YR; j++) { r.ext[j] = sizes[Cfg::yo_id(j)]; r.sin[j] = (int)sYin[Cfg::yo_id(j)]; }
+            hipLaunchKernelGGL(tc_repack_kernel<T>, dim3((unsigned)((ny + 255) / 256)), dim3(256), 0, stream, y, ws + off_y, r);
+            y = ws + off_y;
+        }
+        if (tc_check_launch("repack kernel launch failed") != TC_OK) { (void)hipFreeAsync(ws, stream); return TC_ERR_LAUNCH; }
+    }
+
+    const dim3 g((unsigned)grid), b(Cfg::NT);
     // swapped MFMA roles with 128-bit C accesses: fp32 only, fastest extent a multiple of 4, C 16-byte aligned
     const bool swp = Cfg::SWAP && (sizes[Cfg::c_id(0)] % 4 == 0) && (((uintptr_t)C & 15) == 0);
     tc_launch_variant<Cfg>(nkb == 1, ext_full, int_full, swp, g, b, stream, c, x, y, d);
-    return tc_check_launch("tiled kernel launch failed");
+    const int rc = tc_check_launch("tiled kernel launch failed");
+    if (ws && hipFreeAsync(ws, stream) != hipSuccess) { (void)hipGetLastError(); if (rc == TC_OK) return tc_fail(TC_ERR_ALLOC, "stream-ordered free of the repack buffer failed"); }
+    return rc;
 }
 
 // The reference's calling convention: HOST pointers in, result copied back

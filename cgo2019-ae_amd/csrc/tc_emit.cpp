@@ -43,8 +43,8 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
 {
     std::ostringstream o;
     const char* T = t == DType::F64 ? "double" : "float";
-    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
-    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
+    // the inputs in the memory order the kernel reads them in (tile order for a repacked input)
+    const std::vector<int> xop = operand_order(c, m, true), yop = operand_order(c, m, false);
 
     o << "// Emitted by cogent-mi355 for gfx950.  Do not edit: regenerate from the expression.\n";
     o << "//   " << c.text << "\n";
@@ -87,11 +87,11 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
         o << table((s + "o_id").c_str(), ids) << table((s + "o_tile").c_str(), tiles)
           << table((s + "o_isk").c_str(), isk) << table((s + "o_mul").c_str(), mul);
     };
-    o << "    // the X- and Y-side operands in their own memory order: id, tile, contracted?, weight in the composite coordinate\n";
+    o << "    // the X- and Y-side operands in the memory order the kernel reads: id, tile, contracted?, weight in the composite coordinate\n";
     operand("X", xop, m.x_ids, m.x_tiles);
     operand("Y", yop, m.y_ids, m.y_tiles);
     o << "    static constexpr int WX = " << m.WX << ", WY = " << m.WY << ", TX = " << m.TX << ", TY = " << m.TY << ", NT = " << 64 * m.WX * m.WY << ";\n";
-    o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ";\n";
+    o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ", RPX = " << m.RPX << ", RPY = " << m.RPY << ";\n";
     o << "    static constexpr int LAYX = " << m.layx << ", LDX = " << m.ldx << ", LAYY = " << m.layy << ", LDY = " << m.ldy << ";\n";
     o << "};\n";
     o << "}  // namespace\n\n";

@@ -72,6 +72,7 @@ struct Mapping {
     int swap_forced = -1;
     int PD = 1;                               // K blocks requested ahead of the one being contracted (register stages)
     int pd_forced = -1;
+    int RPX = 0, RPY = 0;                     // 1 (mapping spec rx=/ry= only): that input is first copied into tile order, see operand_order()
     int SK = 1;                               // split-K factor: SK workgroups per output tile, atomic accumulate
     int layx = 0, ldx = 0, layy = 0, ldy = 0; // LDS layout per operand
     // model outputs
@@ -97,6 +98,9 @@ bool select_mapping(const Contraction& c, DType t, const ArchGfx950& arch, int r
 bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, const std::string& spec, Mapping& out, std::string& err);
 bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const Mapping& m, std::string& err);
 std::string mapping_json(const Contraction& c, DType t, const Mapping& m);
+// Index ids of the X-side (or Y-side) input in the memory order the kernel reads it in, fastest first:
+// the tensor's own order, or for a repacked input its externals in tile order followed by the K indices.
+std::vector<int> operand_order(const Contraction& c, const Mapping& m, bool x_side);
 
 // ---- emitter (tc_emit.cpp)
 std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, const std::string& unique_name);

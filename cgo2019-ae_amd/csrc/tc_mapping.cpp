@@ -68,6 +68,8 @@ std::string Mapping::spec() const
     if (ntc_forced >= 0) o << ";nt=" << ntc_forced;
     if (swap_forced >= 0) o << ";sw=" << swap_forced;
     if (pd_forced >= 1) o << ";pd=" << pd_forced;
+    if (RPX) o << ";rx=1";
+    if (RPY) o << ";ry=1";
     return o.str();
 }
 
@@ -167,6 +169,15 @@ static void finish_geometry(const Contraction& c, DType t, Mapping& m)
     // fp32: put C's fastest index on the MFMA rows when its tile is a multiple of 4 (128-bit C accesses)
     const bool can_swap = t == DType::F32 && !m.x_tiles.empty() && m.x_ids[0] == c.out_idx[0] && m.x_tiles[0] % 4 == 0;
     m.SWAP = can_swap && (m.swap_forced != 0) ? 1 : 0;
+}
+
+std::vector<int> operand_order(const Contraction& c, const Mapping& m, bool x_side)
+{
+    const bool is_a = x_side ? m.x_is_a : !m.x_is_a;
+    if (!(x_side ? m.RPX : m.RPY)) return is_a ? c.a_idx : c.b_idx;
+    std::vector<int> o = x_side ? m.x_ids : m.y_ids;
+    o.insert(o.end(), m.k_ids.begin(), m.k_ids.end());
+    return o;
 }
 
 bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const Mapping& m, std::string& err)
@@ -303,8 +314,7 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     m.blocks_per_cu = r;
     const double waves_simd = (double)(r * W) / arch.simd_per_cu;      // resident wavefronts per SIMD
 
-    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
-    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
+    const std::vector<int> xop = operand_order(c, m, true), yop = operand_order(c, m, false);
     // ---- HBM: a streaming kernel reaches the sustained rate only with about four resident
     // wavefronts per SIMD in different phases (load C / contract / store C); measured 0.75 at two
     const double bw = arch.hbm_bytes_per_s * arch.hbm_sustained_fraction;
@@ -353,6 +363,9 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     for (double p : parts) { mx = std::max(mx, p); sum += p; }
     // the slowest pipe sets the pace; the others overlap imperfectly
     m.cost = (mx + 0.15 * (sum - mx)) * spill_penalty / std::max(m.tail_eff, 0.05) + 2.0e-6;
+    // a repacked input is read and written once more by a kernel of its own, which the contraction waits for
+    if (m.RPX) m.cost += 2.0 * nX * s / bw + 4.0e-6;
+    if (m.RPY) m.cost += 2.0 * nY * s / bw + 4.0e-6;
 }
 
 static void wave_layouts(int nx, int ny, int max_acc_tiles, std::vector<std::array<int, 4>>& out)
@@ -543,14 +556,15 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "nt") m.ntc_forced = std::max(0, std::min(3, atoi(val.c_str())));
         else if (key == "sw") m.swap_forced = atoi(val.c_str()) ? 1 : 0;
         else if (key == "pd") m.pd_forced = std::max(1, std::min(8, atoi(val.c_str())));
+        else if (key == "rx") m.RPX = atoi(val.c_str()) ? 1 : 0;
+        else if (key == "ry") m.RPY = atoi(val.c_str()) ? 1 : 0;
         else if (key == "lx") lx = atoi(val.c_str());
         else if (key == "ly") ly = atoi(val.c_str());
         else { err = "mapping spec: unknown key " + key; return false; }
     }
     if (m.MI < 0 || m.MI > 2) { err = "mapping spec: unknown matrix instruction"; return false; }
-    const std::vector<int>& xop = m.x_is_a ? c.a_idx : c.b_idx;
-    const std::vector<int>& yop = m.x_is_a ? c.b_idx : c.a_idx;
     if (m.x_ids.empty()) { err = "mapping spec must give x"; return false; }
+    const std::vector<int> xop = operand_order(c, m, true), yop = operand_order(c, m, false);
     m.layx = lx >= 0 ? lx : ((!m.k_ids.empty() && m.k_ids[0] == fvi(xop) && m.k_tiles[0] >= 4) ? 1 : 0);
     m.layy = ly >= 0 ? ly : ((!m.k_ids.empty() && m.k_ids[0] == fvi(yop) && m.k_tiles[0] >= 4) ? 1 : 0);
     finish_geometry(c, t, m);
@@ -575,7 +589,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

@@ -90,6 +90,10 @@ def test_kernel_options_in_a_spec(tools):
     assert "pd=3" in m["spec"] and "nt=2" in m["spec"]
     again = tools.plan(text, "DOUBLE", mapping_spec=m["spec"]).info["mapping"]
     assert again == m
+    # rx=/ry=: an input copied into tile order first; its slices then go to LDS K-major whatever its own order
+    m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:24,a:2;k=e:12;w=3x1;t=3x3;rx=1;ry=1").info["mapping"]
+    assert m["repack"] == [1, 1] and m["lds_layout"] == [0, 0] and "rx=1" in m["spec"] and "ry=1" in m["spec"]
+    assert tools.plan(text, "DOUBLE").info["mapping"]["repack"] == [0, 0]      # never chosen automatically
     # fp32 with a fastest tile that is a multiple of 4: swapped roles by default, sw=0 turns them off
     text4 = open(os.path.join(EXPR_DIR, "cfg4_16_f32.in")).read()
     auto = tools.plan(text4, "FLOAT").info["mapping"]
