@@ -5,6 +5,10 @@
   generated/<name>.hip     one emitted translation unit per expression in expressions/manifest.json
   lib/<name>.so            the same, compiled for gfx950                                   (hipcc)
   lib/libcogent_driver.so  timing driver (HIP events around batches of launches)           (hipcc)
+  tuning/<name>/cand_NN.so candidate mappings of the entries listed in TUNING_SETS, for the on-GPU tuner
+
+A mapping comes from, in this order: the entry's "map" in manifest.json (pinned by hand), the tuner's
+cache expressions/tuned.json (measured), the mapping pass's cost model.
 
 hipcc cross-compiles for gfx950 without a GPU, so this runs on a CPU-only machine.
 """
@@ -50,13 +54,28 @@ def build_host_tools():
          os.path.join(CSRC, "tc_cli.cpp"), "-L" + LIB, "-lcogent_mi355", "-Wl,-rpath,$ORIGIN/../lib"])
 
 
+# manifest entries whose top candidates are compiled ahead of time so that the tuner's measuring step
+# (cogent_mi355/tuner.py) has something to time on a GPU machine without compiling there
+TUNING_SETS = {"cfg5_1_f64": 3}
+
+
+def tuned_map(entry):
+    path = os.path.join(EXPR, "tuned.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        hit = json.load(f).get("%s|%s|%s" % (entry["file"], entry["dtype"], ",".join(str(s) for s in entry["bench_sizes"])))
+    return hit["map"] if hit else None
+
+
 def emit_and_compile(entry):
     name = entry["name"]
     hip = os.path.join(GEN, name + ".hip")
     cmd = [os.path.join(BIN, "cogent_gen"), name, os.path.join(EXPR, entry["file"]),
            str(entry.get("config", -1)), "-1", entry["dtype"], "-o", hip, "--name", name]
-    if entry.get("map"):
-        cmd += ["--map", entry["map"]]
+    spec = entry.get("map") or tuned_map(entry)
+    if spec:
+        cmd += ["--map", spec]
     run(cmd)
     run(["hipcc"] + HIPCC_FLAGS + ["-o", os.path.join(LIB, name + ".so"), hip])
     return name
@@ -76,6 +95,13 @@ def build_all(jobs=8, only=None):
         futs.append(ex.submit(build_driver))
         for f in futs:
             f.result()
+    if only is None:
+        sys.path.insert(0, HERE)
+        from cogent_mi355 import tuner
+        for name, k in TUNING_SETS.items():
+            bad = [c for c in tuner.prepare(name, k, jobs=jobs) if "so" not in c]
+            if bad:
+                raise RuntimeError("tuning candidate failed to build: %r" % bad[0])
     return [e["name"] for e in entries]
 
 

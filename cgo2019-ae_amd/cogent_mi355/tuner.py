@@ -1,0 +1,180 @@
+"""Measured choice of a mapping: time the model's best candidates on the GPU and cache the winner.
+
+The reference picks its configuration from a cost model alone and offers a manual override by rank
+(cogent/src/generators/configurations.py:254-289).  Here the model ranks the candidates, and this module
+can settle the choice by measurement in two steps that run in different places:
+
+  prepare(name, top_k)   on any machine with hipcc (no GPU needed): emit and compile the model's top_k distinct
+                         candidates of a manifest entry into tuning/<name>/cand_NN.so, with an index file
+  measure(name)          on the GPU: check every candidate against the one-lane-per-element kernel of the same
+                         object, time it with HIP events, and write the winner's mapping spec to
+                         expressions/tuned.json, which build.py honours (below a "map" pinned in manifest.json,
+                         above the model's own choice)
+
+Command line:  python -m cogent_mi355.tuner prepare|measure|show <name> [--top K] [--sizes a,b,...]
+"""
+import argparse
+import concurrent.futures
+import json
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TUNING = os.path.join(HERE, "tuning")
+CACHE = os.path.join(HERE, "expressions", "tuned.json")
+
+
+def _build():
+    sys.path.insert(0, HERE)
+    import build
+    return build
+
+
+def cache_key(entry, sizes=None):
+    return "%s|%s|%s" % (entry["file"], entry["dtype"], ",".join(str(s) for s in (sizes or entry["bench_sizes"])))
+
+
+def load_cache(path=CACHE):
+    if not os.path.exists(path):
+        return {}
+    with open(path) as f:
+        return json.load(f)
+
+
+def distinct_candidates(cands, top_k):
+    """The first top_k candidates that differ in tiles, wavefront grid or instruction (not only in model cost)."""
+    seen, out = set(), []
+    for c in cands:
+        key = (tuple(c["block_tile"]), tuple(c["waves"]), tuple(map(tuple, c["x"])), tuple(map(tuple, c["y"])),
+               tuple(map(tuple, c["k"])), c["mfma"], c["split_k"], tuple(c["lds_layout"]))
+        if key in seen:
+            continue
+        seen.add(key)
+        out.append(c)
+        if len(out) >= top_k:
+            break
+    return out
+
+
+def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
+    """Emit and compile the candidates of manifest entry `name`.  Returns the index (list of dicts)."""
+    b = _build()
+    entry = [e for e in b.manifest() if e["name"] == name][0]
+    gen = os.path.join(b.BIN, "cogent_gen")
+    src = os.path.join(b.EXPR, entry["file"])
+    listing = b.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", os.devnull, "--list", str(max(4 * top_k, 40))])
+    specs = list(extra_specs) + [c["spec"] for c in distinct_candidates(json.loads(listing), top_k)]
+    if entry.get("map") and entry["map"] not in specs:
+        specs.insert(0, entry["map"])                      # the pinned mapping defends its place
+    out = os.path.join(out_root, name)
+    os.makedirs(out, exist_ok=True)
+    for f in os.listdir(out):
+        os.remove(os.path.join(out, f))
+
+    def one(args):
+        i, spec = args
+        hip = os.path.join(out, "cand_%02d.hip" % i)
+        so = os.path.join(out, "cand_%02d.so" % i)
+        r = subprocess.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", hip, "--name", name, "--map", spec],
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if r.returncode:
+            return {"i": i, "spec": spec, "error": "generator: " + r.stdout.strip()}
+        r = subprocess.run(["hipcc"] + b.HIPCC_FLAGS + ["-o", so, hip], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        os.remove(hip)
+        if r.returncode:
+            return {"i": i, "spec": spec, "error": "hipcc: " + r.stdout[-400:]}
+        return {"i": i, "spec": spec, "so": os.path.basename(so)}
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        index = list(ex.map(one, enumerate(specs)))
+    with open(os.path.join(out, "index.json"), "w") as f:
+        json.dump({"name": name, "file": entry["file"], "dtype": entry["dtype"], "candidates": index}, f, indent=1)
+    return index
+
+
+def measure(name, sizes=None, warmup=3, iters=20, out_root=TUNING, cache_path=CACHE, tol=None):
+    """Verify and time the prepared candidates on the GPU; record the fastest correct one.  Returns a report."""
+    import numpy as np
+    import torch
+    import cogent_mi355 as pkg
+    with open(os.path.join(out_root, name, "index.json")) as f:
+        idx = json.load(f)
+    entry = pkg.manifest_entry(name)
+    sizes = [int(s) for s in (sizes or entry["bench_sizes"])]
+    tools, driver = pkg.HostTools(), pkg.Driver()
+    plan = tools.plan(open(os.path.join(HERE, "expressions", idx["file"])).read(), idx["dtype"])
+    dtype = torch.float64 if idx["dtype"] == "DOUBLE" else torch.float32
+    tol = tol if tol is not None else (1e-12 if idx["dtype"] == "DOUBLE" else 1e-5)
+    info = plan.info
+    ext = dict(zip(info["out_idx"] + info["sum_idx"], sizes))
+    count = lambda names: int(np.prod([ext[n] for n in names], dtype=np.int64))
+    nC, nA, nB = count(info["out_idx"]), count(info["a_idx"]), count(info["b_idx"])
+    g = torch.Generator(device="cuda").manual_seed(1)
+    A = torch.rand(nA, dtype=dtype, device="cuda", generator=g) * 2 - 1
+    B = torch.rand(nB, dtype=dtype, device="cuda", generator=g) * 2 - 1
+    C0 = torch.rand(nC, dtype=dtype, device="cuda", generator=g) * 2 - 1
+    # enough output buffers that the Infinity Cache (256 MB) cannot hold them between launches
+    nbuf = max(2, min(16, int(1.2e9 // max(1, nC * C0.element_size())) + 1))
+    bufs = [C0.clone() for _ in range(nbuf)]
+    rows, want = [], None
+    for cand in idx["candidates"]:
+        if "so" not in cand:
+            rows.append(dict(cand, ok=False))
+            continue
+        ex = pkg.Expression(path=os.path.join(out_root, name, cand["so"]))
+        if want is None:                                   # the reference result: the plain kernel, once
+            want = C0.clone()
+            rc = ex.run(sizes, want.data_ptr(), A.data_ptr(), B.data_ptr(), None, 1)
+            torch.cuda.synchronize()
+            if rc:
+                raise pkg.CogentError("plain kernel failed: " + ex.last_error())
+            scale = torch.maximum(want.abs(), want.pow(2).mean().sqrt())
+        got = C0.clone()
+        rc = ex.entry(sizes, got.data_ptr(), A.data_ptr(), B.data_ptr())
+        torch.cuda.synchronize()
+        err = float(((got - want).abs() / scale).max()) if rc == 0 else float("inf")
+        row = dict(cand, status=rc, max_rel_err=err, ok=(rc == 0 and err <= tol))
+        if row["ok"]:
+            st = driver.time(ex, sizes, [b_.data_ptr() for b_ in bufs], A.data_ptr(), B.data_ptr(), warmup, iters)
+            row.update(mean_us=st["mean_ms"] * 1e3, min_us=st["min_ms"] * 1e3, model_us=ex.info["model"]["cost_us"])
+        rows.append(row)
+    good = [r for r in rows if r.get("ok")]
+    report = {"name": name, "sizes": sizes, "candidates": rows, "best": None}
+    if good:
+        best = min(good, key=lambda r: r["mean_us"])
+        report["best"] = {"spec": best["spec"], "mean_us": best["mean_us"]}
+        cache = load_cache(cache_path)
+        cache[cache_key(entry, sizes)] = {"map": best["spec"], "mean_us": round(best["mean_us"], 2),
+                                          "candidates_timed": len(good)}
+        with open(cache_path, "w") as f:
+            json.dump(cache, f, indent=1, sort_keys=True)
+    return report
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("step", choices=["prepare", "measure", "show"])
+    ap.add_argument("name", help="entry of expressions/manifest.json")
+    ap.add_argument("--top", type=int, default=6)
+    ap.add_argument("--sizes", default="")
+    ap.add_argument("--spec", action="append", default=[], help="an extra mapping spec to include (repeatable)")
+    a = ap.parse_args(argv)
+    sizes = [int(s) for s in a.sizes.split(",")] if a.sizes else None
+    if a.step == "prepare":
+        for c in prepare(a.name, a.top, a.spec):
+            print("%02d %s %s" % (c["i"], "built " if "so" in c else "FAILED", c.get("error", c["spec"])))
+    elif a.step == "measure":
+        rep = measure(a.name, sizes)
+        for r in sorted(rep["candidates"], key=lambda r: r.get("mean_us", 1e30)):
+            print("%10s us  model %8s  err %-9s %s" % ("%.1f" % r["mean_us"] if "mean_us" in r else "-",
+                  "%.1f" % r["model_us"] if "model_us" in r else "-", "%.1e" % r["max_rel_err"] if "max_rel_err" in r else "-", r["spec"]))
+        print("best:", rep["best"])
+    else:
+        b = _build()
+        entry = [e for e in b.manifest() if e["name"] == a.name][0]
+        print(load_cache().get(cache_key(entry, sizes)))
+
+
+if __name__ == "__main__":
+    main()

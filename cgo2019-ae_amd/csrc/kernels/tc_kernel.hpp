@@ -179,7 +179,9 @@ __device__ __forceinline__ void slice_store(const typename Cfg::T (&reg)[SLOTS],
 // Normal roles (X along MFMA columns): cx[tj][0] for the lane's column in tile column tj, cy[ti][r] for
 // the row of register r in tile row ti.  Swapped roles (SWP, X along MFMA rows): cx[tj][r], cy[ti][0].
 // -1 marks positions outside the tensor (ragged tiles, padding).
-template <class Cfg, bool EXT_FULL, bool SWP>
+// LOCAL: the offsets are positions in a dense copy of the tile alone, kept in C's index order (the
+// layout of the tile when it is staged through LDS), instead of offsets into the tensor.
+template <class Cfg, bool EXT_FULL, bool SWP, bool LOCAL>
 __device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const int* rem, const TcDims& d,
                                                int (&cx)[Cfg::TX][SWP ? Mfma<Cfg::MI>::NREG : 1],
                                                int (&cy)[Cfg::TY][SWP ? 1 : Mfma<Cfg::MI>::NREG])
@@ -197,7 +199,7 @@ __device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const i
             for (int i = 0; i < Cfg::NX; i++) {
                 const int c = (int)(q % (unsigned)Cfg::x_tile(i));
                 q /= (unsigned)Cfg::x_tile(i);
-                off += c * d.sC[Cfg::x_id(i)];
+                off += c * (LOCAL ? Cfg::cl_stride(Cfg::x_id(i)) : d.sC[Cfg::x_id(i)]);
                 if (!EXT_FULL) ok = ok && (c < rem[Cfg::x_id(i)]);
             }
             cx[tj][r] = ok ? off : -1;
@@ -214,7 +216,7 @@ __device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const i
             for (int i = 0; i < Cfg::NY; i++) {
                 const int c = (int)(q % (unsigned)Cfg::y_tile(i));
                 q /= (unsigned)Cfg::y_tile(i);
-                off += c * d.sC[Cfg::y_id(i)];
+                off += c * (LOCAL ? Cfg::cl_stride(Cfg::y_id(i)) : d.sC[Cfg::y_id(i)]);
                 if (!EXT_FULL) ok = ok && (c < rem[Cfg::y_id(i)]);
             }
             cy[ti][r] = ok ? off : -1;
@@ -272,8 +274,18 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     // written while other wavefronts still read the current ones, one barrier per K block
     constexpr int NBUF = (!ONE_KB && 2 * (LDS_X + LDS_Y) * (int)sizeof(T) <= 65536) ? 2 : 1;
 
-    __shared__ T lds_x_all[NBUF * LDS_X];
-    __shared__ T lds_y_all[NBUF * LDS_Y];
+    // C tile through LDS (CL): the tile is read from and written to global memory in C's own memory
+    // order, 16 bytes per lane and whole lines per wavefront whatever the MFMA lane layout is, and
+    // changes hands with the accumulators through a dense copy in LDS that shares the operand buffers.
+    // Full tiles without split K only; the other variants of the same object use the direct path.
+    constexpr int SK0 = ONE_KB ? 1 : Cfg::SK;
+    constexpr bool CL = (Cfg::CLDS != 0) && EXT_FULL && SK0 == 1 && (ONE_KB || Cfg::LATEC == 0);
+    constexpr int TILE_VOL = Cfg::BX * Cfg::BY;
+    constexpr int LDS_OPS = NBUF * (LDS_X + LDS_Y);
+    constexpr int LDS_ALL = (CL && TILE_VOL > LDS_OPS) ? TILE_VOL : LDS_OPS;
+    __shared__ __attribute__((aligned(16))) T lds_all[LDS_ALL];
+    T* const lds_x_all = lds_all;
+    T* const lds_y_all = lds_all + NBUF * LDS_X;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -340,8 +352,8 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     // ---- where this lane's accumulator elements live in C (-1: outside)
     int cx[TX][SWP ? NREG : 1];
     int cy[TY][SWP ? 1 : NREG];
-    c_tile_offsets<Cfg, EXT_FULL, SWP>(lane, wx, wy, rem, d, cx, cy);
-    // offset of accumulator element (ti, tj, r) and whether it is inside the tensor
+    c_tile_offsets<Cfg, EXT_FULL, SWP, CL>(lane, wx, wy, rem, d, cx, cy);
+    // offset of accumulator element (ti, tj, r) (CL: its place in the LDS copy) and whether it is inside the tensor
     auto c_off = [&](int ti, int tj, int r) -> int { return cx[tj][SWP ? r : 0] + cy[ti][SWP ? 0 : r]; };
     auto c_ok = [&](int ti, int tj, int r) -> bool {
         return (EXT_FULL && !PADDED) || (cx[tj][SWP ? r : 0] >= 0 && cy[ti][SWP ? 0 : r] >= 0);
@@ -357,6 +369,35 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     constexpr bool LATE_C = !ONE_KB && SK == 1 && (Cfg::LATEC != 0);
     Acc cpre[LATE_C ? TY : 1][LATE_C ? TX : 1];
     Acc acc[TY][TX];
+    // the tile in C's memory order: element q of it, as an offset from the tile origin
+    constexpr int CV = 16 / (int)sizeof(T);
+    typedef T TV __attribute__((ext_vector_type(CV)));
+    constexpr int NVEC = CL ? (TILE_VOL / CV + NT - 1) / NT : 1;
+    auto c_linear = [&](unsigned q) -> unsigned {
+        unsigned off = 0;
+#pragma unroll
+        for (int j = 0; j < Cfg::CR; j++) {
+            const unsigned t = (unsigned)Cfg::c_tile(j);
+            off += (q % t) * (unsigned)d.sC[Cfg::c_id(j)];
+            q /= t;
+        }
+        return off;
+    };
+    if (CL) {
+        TV cv[NVEC];
+#pragma unroll
+        for (int i = 0; i < NVEC; i++) {
+            const unsigned q = (unsigned)(tid + i * NT) * CV;
+            if (TILE_VOL % (NT * CV) == 0 || q < (unsigned)TILE_VOL)
+                cv[i] = c_load<(Cfg::NTC & 1) != 0>((const TV*)(Cb + c_linear(q)));
+        }
+#pragma unroll
+        for (int i = 0; i < NVEC; i++) {
+            const unsigned q = (unsigned)(tid + i * NT) * CV;
+            if (TILE_VOL % (NT * CV) == 0 || q < (unsigned)TILE_VOL) *(TV*)&lds_all[q] = cv[i];
+        }
+        __syncthreads();
+    }
 #pragma unroll
     for (int ti = 0; ti < TY; ti++)
 #pragma unroll
@@ -365,8 +406,10 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
                 for (int g = 0; g < NREG / 4; g++) {
                     T4 v = {(T)0, (T)0, (T)0, (T)0};
-                    if (SK == 1 && !LATE_C && c_ok(ti, tj, 4 * g))
-                        v = c_load<(Cfg::NTC & 1) != 0>((const T4*)((const char*)Cb + (unsigned)c_off(ti, tj, 4 * g) * (unsigned)sizeof(T)));
+                    if (SK == 1 && !LATE_C && c_ok(ti, tj, 4 * g)) {
+                        if (CL) v = *(const T4*)&lds_all[c_off(ti, tj, 4 * g)];
+                        else v = c_load<(Cfg::NTC & 1) != 0>((const T4*)((const char*)Cb + (unsigned)c_off(ti, tj, 4 * g) * (unsigned)sizeof(T)));
+                    }
 #pragma unroll
                     for (int e = 0; e < 4; e++) acc[ti][tj][4 * g + e] = v[e];
                 }
@@ -374,12 +417,15 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
 #pragma unroll
                 for (int r = 0; r < NREG; r++) {
                     T v = (T)0;
-                    if (SK == 1 && !LATE_C && c_ok(ti, tj, r))
-                        v = c_load<(Cfg::NTC & 1) != 0>((const T*)((const char*)Cb + (unsigned)c_off(ti, tj, r) * (unsigned)sizeof(T)));
+                    if (SK == 1 && !LATE_C && c_ok(ti, tj, r)) {
+                        if (CL) v = lds_all[c_off(ti, tj, r)];
+                        else v = c_load<(Cfg::NTC & 1) != 0>((const T*)((const char*)Cb + (unsigned)c_off(ti, tj, r) * (unsigned)sizeof(T)));
+                    }
                     acc[ti][tj][r] = v;
                 }
             }
         }
+    if (CL) __syncthreads();        // the copy has been read: the operand slices may take its place
 
     // ---- padding rows/columns of the LDS slices are never written by the staging: clear once
     if (PADDED) {
@@ -538,7 +584,37 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     if (!ONE_KB) {
         int lane2 = lane;
         asm volatile("" : "+v"(lane2));
-        c_tile_offsets<Cfg, EXT_FULL, SWP>(lane2, wx, wy, rem, d, cx, cy);
+        c_tile_offsets<Cfg, EXT_FULL, SWP, CL>(lane2, wx, wy, rem, d, cx, cy);
+    }
+    if (CL) {
+        __syncthreads();            // every wavefront is done with the operand slices
+#pragma unroll
+        for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+            for (int tj = 0; tj < TX; tj++) {
+                if (VEC4) {
+#pragma unroll
+                    for (int g = 0; g < NREG / 4; g++)
+                        if (c_ok(ti, tj, 4 * g)) {
+                            T4 v;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) v[e] = acc[ti][tj][4 * g + e];
+                            *(T4*)&lds_all[c_off(ti, tj, 4 * g)] = v;
+                        }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < NREG; r++)
+                        if (c_ok(ti, tj, r)) lds_all[c_off(ti, tj, r)] = acc[ti][tj][r];
+                }
+            }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NVEC; i++) {
+            const unsigned q = (unsigned)(tid + i * NT) * CV;
+            if (TILE_VOL % (NT * CV) == 0 || q < (unsigned)TILE_VOL)
+                c_store<(Cfg::NTC & 2) != 0>(*(const TV*)&lds_all[q], (TV*)(Cb + c_linear(q)));
+        }
+        return;
     }
 #pragma unroll
     for (int ti = 0; ti < TY; ti++)

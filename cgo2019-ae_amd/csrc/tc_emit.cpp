@@ -63,6 +63,20 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
     o << table("x_id", m.x_ids) << table("x_tile", m.x_tiles);
     o << table("y_id", m.y_ids) << table("y_tile", m.y_tiles);
     o << table("k_id", m.k_ids) << table("k_tile", m.k_tiles);
+    {
+        // the C tile as a dense block in C's own index order: tile per C index, stride per index id
+        std::vector<int> ct, cls(c.n_idx(), 0);
+        int run = 1;
+        for (int id : c.out_idx) {
+            int p, tl = 1;
+            if ((p = pos_in(m.x_ids, id)) >= 0) tl = m.x_tiles[p];
+            else if ((p = pos_in(m.y_ids, id)) >= 0) tl = m.y_tiles[p];
+            ct.push_back(tl);
+            cls[id] = run;
+            run *= tl;
+        }
+        o << table("c_tile", ct) << table("cl_stride", cls);
+    }
     o << "    static constexpr int BX = " << m.BX << ", BY = " << m.BY << ", BK = " << m.BK << ";\n";
     o << "    static constexpr int BXP = " << m.BXP << ", BYP = " << m.BYP << ", BKP = " << m.BKP << ";\n";
 
@@ -91,7 +105,7 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
     operand("X", xop, m.x_ids, m.x_tiles);
     operand("Y", yop, m.y_ids, m.y_tiles);
     o << "    static constexpr int WX = " << m.WX << ", WY = " << m.WY << ", TX = " << m.TX << ", TY = " << m.TY << ", NT = " << 64 * m.WX * m.WY << ";\n";
-    o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ", RPX = " << m.RPX << ", RPY = " << m.RPY << ";\n";
+    o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ", RPX = " << m.RPX << ", RPY = " << m.RPY << ", CLDS = " << m.CLDS << ";\n";
     o << "    static constexpr int LAYX = " << m.layx << ", LDX = " << m.ldx << ", LAYY = " << m.layy << ", LDY = " << m.ldy << ";\n";
     o << "};\n";
     o << "}  // namespace\n\n";

@@ -73,6 +73,8 @@ struct Mapping {
     int PD = 1;                               // K blocks requested ahead of the one being contracted (register stages)
     int pd_forced = -1;
     int RPX = 0, RPY = 0;                     // 1 (mapping spec rx=/ry= only): that input is first copied into tile order, see operand_order()
+    int CLDS = 0;                             // 1: full C tiles pass through LDS in C's memory order (16-byte, whole-line global accesses)
+    int clds_forced = -1;
     int SK = 1;                               // split-K factor: SK workgroups per output tile, atomic accumulate
     int layx = 0, ldx = 0, layy = 0, ldy = 0; // LDS layout per operand
     // model outputs

@@ -68,6 +68,7 @@ std::string Mapping::spec() const
     if (ntc_forced >= 0) o << ";nt=" << ntc_forced;
     if (swap_forced >= 0) o << ";sw=" << swap_forced;
     if (pd_forced >= 1) o << ";pd=" << pd_forced;
+    if (clds_forced >= 0) o << ";cl=" << clds_forced;
     if (RPX) o << ";rx=1";
     if (RPY) o << ";ry=1";
     return o.str();
@@ -274,7 +275,20 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
         chunk *= tl;
         if (tl != c.indices[id].rep_size) break;
     }
-    const double c_hbm_eff = std::min(1.0, chunk * s / 128.0);
+    // C through LDS (mapping spec cl=1 only): possible for 16-byte multiples along C's fastest index,
+    // tiles of at most 64 KB, no split K.  The tile is then moved in its own memory order with 16-byte
+    // accesses, a contiguous kilobyte per wavefront instruction, non-temporal when it is made of whole
+    // lines.  Measured on config 4 (96-byte rows, 2304-byte planes) and on the TCCG 6-D shapes it
+    // changed nothing (+-2 %), on config 5 it cost 12 %: never chosen automatically.
+    {
+        const double tile_bytes = (double)m.BX * m.BY * s;
+        const bool possible = ((long long)(tile_of(c.out_idx[0]) * s) % 16 == 0) && tile_bytes <= 65536.0 && m.SK == 1 &&
+                              !(m.LATEC && nkb > 1);
+        const bool whole_lines = chunk * s >= 256.0 && std::fmod(chunk * s, 128.0) == 0.0;
+        m.CLDS = (m.clds_forced == 1 && possible) ? 1 : 0;
+        if (m.CLDS && m.ntc_forced < 0) m.NTC = whole_lines ? 3 : 0;
+    }
+    const double c_hbm_eff = m.CLDS ? 1.0 : std::min(1.0, chunk * s / 128.0);
     // address span of the block's C tile relative to its volume: compact tiles keep DRAM pages and
     // TLB entries busy with fewer blocks (measured: tiling the Y side in C's own index order beats
     // the operand's order by 20-40% on the 6-D contractions)
@@ -306,7 +320,7 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const double spill_penalty = regs > reg_cap ? 1.0 + 2.0 * (double)(regs - reg_cap) / reg_cap : 1.0;
     int waves_per_simd = std::max(1, std::min(8, arch.vgpr_per_lane / std::max(regs, 64)));
     const bool two_stage = nkb > 1 && 2 * m.lds_bytes <= arch.lds_bytes_per_block;
-    const int lds_block = m.lds_bytes * (two_stage ? 2 : 1);
+    const int lds_block = std::max(m.lds_bytes * (two_stage ? 2 : 1), m.CLDS ? (int)(m.BX * m.BY * s) : 0);
     int r = std::min(arch.lds_bytes_per_cu / std::max(lds_block, 1), arch.max_waves_per_cu / W);
     r = std::min(r, std::max(1, waves_per_simd * arch.simd_per_cu / W));
     r = std::max(r, 1);
@@ -556,6 +570,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "nt") m.ntc_forced = std::max(0, std::min(3, atoi(val.c_str())));
         else if (key == "sw") m.swap_forced = atoi(val.c_str()) ? 1 : 0;
         else if (key == "pd") m.pd_forced = std::max(1, std::min(8, atoi(val.c_str())));
+        else if (key == "cl") m.clds_forced = atoi(val.c_str()) ? 1 : 0;
         else if (key == "rx") m.RPX = atoi(val.c_str()) ? 1 : 0;
         else if (key == "ry") m.RPY = atoi(val.c_str()) ? 1 : 0;
         else if (key == "lx") lx = atoi(val.c_str());
@@ -589,7 +604,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

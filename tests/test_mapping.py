@@ -94,6 +94,10 @@ def test_kernel_options_in_a_spec(tools):
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:24,a:2;k=e:12;w=3x1;t=3x3;rx=1;ry=1").info["mapping"]
     assert m["repack"] == [1, 1] and m["lds_layout"] == [0, 0] and "rx=1" in m["spec"] and "ry=1" in m["spec"]
     assert tools.plan(text, "DOUBLE").info["mapping"]["repack"] == [0, 0]      # never chosen automatically
+    # cl=1: the C tile passes through LDS in memory order (opt-in; refused silently when the tile is too large)
+    m = tools.plan(text, "DOUBLE", mapping_spec="x=d:8,c:8;y=b:24,a:2;k=e:8;w=2x1;t=2x3;cl=1").info["mapping"]
+    assert m["c_through_lds"] == 1 and "cl=1" in m["spec"]
+    assert tools.plan(text, "DOUBLE", mapping_spec=base + ";cl=1").info["mapping"]["c_through_lds"] == 0   # 96x96x8 B > 64 KB
     # fp32 with a fastest tile that is a multiple of 4: swapped roles by default, sw=0 turns them off
     text4 = open(os.path.join(EXPR_DIR, "cfg4_16_f32.in")).read()
     auto = tools.plan(text4, "FLOAT").info["mapping"]

@@ -1,0 +1,63 @@
+"""The measured-mapping tuner (cogent_mi355/tuner.py): candidate selection, the cache file and its place in the
+build's order of precedence run on the CPU; the measuring step runs on the GPU against candidates the build
+compiled ahead of time.  The reference's counterpart is the rank override of its cost-model choice
+(cogent/src/generators/configurations.py:285-289)."""
+import json
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "cgo2019-ae_amd"))
+
+
+def test_distinct_candidates_skip_repeats_of_one_tiling():
+    from cogent_mi355 import tuner
+    base = {"block_tile": [96, 96, 8], "waves": [2, 2], "x": [["d", 24]], "y": [["b", 24]], "k": [["e", 8]],
+            "mfma": "v_mfma_f64_16x16x4_f64", "split_k": 1, "lds_layout": [0, 0]}
+    cands = [dict(base, spec="a"), dict(base, spec="a2"), dict(base, waves=[4, 1], spec="b"), dict(base, split_k=2, spec="c")]
+    assert [c["spec"] for c in tuner.distinct_candidates(cands, 5)] == ["a", "b", "c"]
+    assert [c["spec"] for c in tuner.distinct_candidates(cands, 2)] == ["a", "b"]
+
+
+def test_prepared_set_of_the_build_is_complete():
+    """build.py compiles the candidates of its TUNING_SETS; the index names one shared object per candidate."""
+    import build
+    for name, k in build.TUNING_SETS.items():
+        d = os.path.join(ROOT, "cgo2019-ae_amd", "tuning", name)
+        idx = json.load(open(os.path.join(d, "index.json")))
+        assert idx["name"] == name and len(idx["candidates"]) >= k
+        for c in idx["candidates"]:
+            assert "error" not in c and os.path.exists(os.path.join(d, c["so"]))
+        assert len({c["spec"] for c in idx["candidates"]}) == len(idx["candidates"])
+
+
+def test_build_prefers_pinned_then_tuned_then_model(tmp_path, monkeypatch):
+    import build
+    from cogent_mi355 import tuner
+    entry = {"name": "x", "file": "cfg5_1_f64.in", "dtype": "DOUBLE", "bench_sizes": [16] * 7}
+    monkeypatch.setattr(build, "EXPR", str(tmp_path))
+    assert build.tuned_map(entry) is None                                   # no cache file
+    key = tuner.cache_key(entry)
+    assert key == "cfg5_1_f64.in|DOUBLE|16,16,16,16,16,16,16"
+    (tmp_path / "tuned.json").write_text(json.dumps({key: {"map": "x=0:16;w=1x1", "mean_us": 1.0}}))
+    assert build.tuned_map(entry) == "x=0:16;w=1x1"
+    assert build.tuned_map(dict(entry, bench_sizes=[24] * 7)) is None       # other sizes: other key
+    assert tuner.load_cache(str(tmp_path / "tuned.json"))[key]["map"] == "x=0:16;w=1x1"
+
+
+@pytest.mark.gpu
+def test_measure_times_verified_candidates_and_records_the_fastest(tmp_path):
+    from cogent_mi355 import tuner
+    cache = str(tmp_path / "tuned.json")
+    print("[gpu] tuner.measure cfg5_1_f64", flush=True)
+    rep = tuner.measure("cfg5_1_f64", warmup=2, iters=10, cache_path=cache)
+    rows = rep["candidates"]
+    assert len(rows) >= 3 and all(r["ok"] for r in rows), rows
+    assert all(r["max_rel_err"] <= 1e-12 for r in rows)
+    best = min(rows, key=lambda r: r["mean_us"])
+    assert rep["best"]["spec"] == best["spec"]
+    assert 20.0 < best["mean_us"] < 500.0                                   # 269 MB of traffic: tens of microseconds
+    saved = json.load(open(cache))
+    assert saved["cfg5_1_f64.in|DOUBLE|16,16,16,16,16,16,16"]["map"] == best["spec"]
