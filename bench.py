@@ -157,7 +157,7 @@ def main():
     ap.add_argument("--only-headline", action="store_true", help="skip the table of the other BASELINE configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
     ap.add_argument("--workload", default=HEADLINE, help="expression object to use as the headline workload")
-    ap.add_argument("--suite", default="", help="'tccg': time the 48 TCCG contractions at the sizes of the reference's "
+    ap.add_argument("--suite", default="", help="'fused': time the fused groups of the manifest; 'tccg': time the 48 TCCG contractions at the sizes of the reference's "
                     "bench script (cogent/bench_tccg.sh:5-54) and print one JSON line with the table, instead of the headline run")
     ap.add_argument("--copy-only", type=int, default=0, metavar="BYTES",
                     help="only run the plain device-to-device copy kernel on BYTES bytes, --steps times "
@@ -182,6 +182,48 @@ def main():
         ms = driver.time_copy(src.data_ptr(), dst.data_ptr(), args.copy_only, args.warmup, args.steps)
         print(json.dumps({"copy_bytes": args.copy_only, "ms_per_copy": ms,
                           "GBps_read_plus_write": round(2 * args.copy_only / ms / 1e6, 1)}))
+        return
+
+    if args.suite == "fused":
+        # fused groups: N contractions into one output in ONE kernel.  Algorithmic bytes: every input once,
+        # the output read once and written once -- not once per term.
+        import numpy as np
+        rows = []
+        for e in pkg.group_manifest():
+            g = pkg.Group(e["name"])
+            sizes = e["bench_sizes"]
+            np_dtype = np.float64 if g.dtype == "f64" else np.float32
+            esz = 8 if g.dtype == "f64" else 4
+            ext = dict(zip(g.info["out_idx"] + g.info["sum_idx"], sizes))
+            count = lambda names: int(np.prod([ext[n] for n in names], dtype=np.int64))
+            nC = count(g.info["out_idx"])
+            dev, in_elems = [], 0
+            for k, term in enumerate(g.info["terms"]):
+                m = term["mapping"]
+                names = {"x": [n for n, _ in m["x"]] + [n for n, _ in m["k"]], "y": [n for n, _ in m["y"]] + [n for n, _ in m["k"]]}
+                x_is_a = (m["x_operand"] == term["text"].split("*")[1].split("[")[0].strip())
+                for which in ((0, 1) if x_is_a else (1, 0)):
+                    n = count(names["x" if which == 0 else "y"])
+                    in_elems += n
+                    dev.append(torch.from_numpy(tools.fill_uniform(np.empty(n, np_dtype), 10 + len(dev))).cuda())
+            n_rot = max(2, min(8, int(1.2e9 // (nC * esz)) + 1))
+            cbufs = [torch.zeros(nC, dtype=torch.float64 if g.dtype == "f64" else torch.float32, device="cuda") for _ in range(n_rot)]
+            st = driver.time_group(g, sizes, [c.data_ptr() for c in cbufs], [d.data_ptr() for d in dev], 3, max(5, min(args.steps, 50)))
+            flops = 2 * int(np.prod(sizes, dtype=np.int64)) * g.n_terms
+            nbytes = esz * (in_elems + 2 * nC)
+            sec = st["mean_ms"] * 1e-3
+            rows.append({"name": e["name"], "sizes": sizes, "dtype": g.dtype, "n_terms": g.n_terms, "flops": flops, "algorithmic_bytes": nbytes,
+                         "bytes_if_run_term_by_term": esz * (in_elems + 2 * nC * g.n_terms),
+                         "kernel_us_mean": round(st["mean_ms"] * 1e3, 2), "kernel_us_min": round(st["min_ms"] * 1e3, 2),
+                         "gflops": round(flops / sec / 1e9, 1),
+                         "roofline": {"bound": "hbm", "achieved": round(nbytes / sec / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                      "frac": round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)},
+                         "roofline_other": {"bound": "mfma", "achieved": round(flops / sec / 1e12, 3), "peak": MFMA_PEAK_TFLOPS[g.dtype],
+                                            "unit": "TFLOP/s", "frac": round(flops / sec / 1e12 / MFMA_PEAK_TFLOPS[g.dtype], 4)},
+                         "c_tile": g.info["c_tile"]})
+            print("%-16s %s  %d terms  %8.1f us  %9.1f GFLOP/s" % (e["name"], sizes, g.n_terms, st["mean_ms"] * 1e3, flops / sec / 1e9),
+                  file=sys.stderr, flush=True)
+        print(json.dumps({"suite": "fused", "unit": "GFLOP/s", "n_gpus": 1, "data": "synthetic", "rows": rows}))
         return
 
     if args.suite:

@@ -44,10 +44,16 @@ def manifest():
         return json.load(f)["expressions"]
 
 
+def group_manifest():
+    """Files that hold several expressions with one output: each becomes one fused-group object."""
+    with open(os.path.join(EXPR, "manifest.json")) as f:
+        return json.load(f).get("groups", [])
+
+
 def build_host_tools():
     os.makedirs(LIB, exist_ok=True)
     os.makedirs(BIN, exist_ok=True)
-    srcs = [os.path.join(CSRC, f) for f in ("tc_parse.cpp", "tc_mapping.cpp", "tc_emit.cpp", "tc_capi.cpp")]
+    srcs = [os.path.join(CSRC, f) for f in ("tc_parse.cpp", "tc_mapping.cpp", "tc_emit.cpp", "tc_group.cpp", "tc_capi.cpp")]
     run(["g++", "-O2", "-std=c++17", "-fopenmp", "-shared", "-fPIC", "-Wall",
          "-o", os.path.join(LIB, "libcogent_mi355.so")] + srcs)
     run(["g++", "-O2", "-std=c++17", "-Wall", "-o", os.path.join(BIN, "cogent_gen"),
@@ -89,7 +95,7 @@ def build_driver():
 def build_all(jobs=8, only=None):
     build_host_tools()
     os.makedirs(GEN, exist_ok=True)
-    entries = [e for e in manifest() if only is None or e["name"] in only]
+    entries = [e for e in manifest() + group_manifest() if only is None or e["name"] in only]
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         futs = [ex.submit(emit_and_compile, e) for e in entries]
         futs.append(ex.submit(build_driver))

@@ -46,8 +46,13 @@ def manifest():
         return json.load(f)["expressions"]
 
 
+def group_manifest():
+    with open(os.path.join(EXPR_DIR, "manifest.json")) as f:
+        return json.load(f).get("groups", [])
+
+
 def manifest_entry(name):
-    for e in manifest():
+    for e in manifest() + group_manifest():
         if e["name"] == name:
             return e
     raise KeyError(name)
@@ -191,6 +196,54 @@ class Expression:
         return self.lib.cogent_run(arr, len(sizes), c_ptr, a_ptr, b_ptr, stream, variant)
 
 
+class Group:
+    """One compiled fused-group object: several contractions into one output, one kernel (lib/<name>.so)."""
+
+    def __init__(self, name=None, path=None):
+        self.path = path or os.path.join(LIB_DIR, name + ".so")
+        self.lib = _load(self.path, hip=True)
+        for fn in (self.lib.cogent_num_indices, self.lib.cogent_num_terms):
+            fn.restype = ctypes.c_int
+        for fn in (self.lib.cogent_last_error, self.lib.cogent_expression, self.lib.cogent_info):
+            fn.restype = ctypes.c_char_p
+        self.n = self.lib.cogent_num_indices()
+        self.n_terms = self.lib.cogent_num_terms()
+        for fn in (self.lib.sd_t_d2_fusion_, self.lib.sd_t_d2_fusion_host_):
+            fn.argtypes = [ctypes.c_int] * self.n + [ctypes.c_void_p] * (1 + 2 * self.n_terms) + [ctypes.c_int] * (self.n_terms + 1)
+            fn.restype = ctypes.c_int
+        self.lib.cogent_run_group.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_void_p,
+                                              ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.c_void_p]
+        self.lib.cogent_run_group.restype = ctypes.c_int
+        self.expressions = self.lib.cogent_expression().decode().split("\n")
+        self.info = json.loads(self.lib.cogent_info().decode())
+        self.dtype = self.info["dtype"]
+
+    def last_error(self):
+        return self.lib.cogent_last_error().decode()
+
+    def _check(self, sizes, inputs):
+        if len(sizes) != self.n:
+            raise CogentError("expected %d extents, got %d" % (self.n, len(sizes)))
+        if len(inputs) != 2 * self.n_terms:
+            raise CogentError("expected %d input pointers, got %d" % (2 * self.n_terms, len(inputs)))
+
+    def entry(self, sizes, c_ptr, inputs, enabled=None):
+        """sd_t_d2_fusion_(size..., C, A1, B1, ..., AN, BN, cond_1..cond_N, -1) on device addresses."""
+        self._check(sizes, inputs)
+        flags = [1] * self.n_terms if enabled is None else [int(bool(v)) for v in enabled]
+        return self.lib.sd_t_d2_fusion_(*[int(s) for s in sizes], c_ptr, *inputs, *flags, -1)
+
+    def entry_host(self, sizes, c_ptr, inputs):
+        self._check(sizes, inputs)
+        return self.lib.sd_t_d2_fusion_host_(*[int(s) for s in sizes], c_ptr, *inputs, *([1] * self.n_terms), -1)
+
+    def run(self, sizes, c_ptr, inputs, enabled=None, stream=None):
+        arr = (ctypes.c_int * len(sizes))(*[int(s) for s in sizes])
+        ptrs = (ctypes.c_void_p * len(inputs))(*inputs)
+        en = None if enabled is None else (ctypes.c_int * len(enabled))(*[int(bool(v)) for v in enabled])
+        return self.lib.cogent_run_group(arr, len(sizes), c_ptr, ptrs, len(inputs), en, stream)
+
+
 class Driver:
     """libcogent_driver.so: HIP-event timing of a loaded expression object."""
 
@@ -214,6 +267,23 @@ class Driver:
         stats = (ctypes.c_float * 4)()
         rc = self.lib.cogent_driver_time(expr.path.encode(), arr, len(sizes), cb, len(c_ptrs), a_ptr, b_ptr,
                                          warmup, iters, variant, each, stats)
+        if rc:
+            raise CogentError("timing failed (%d): %s" % (rc, self.lib.cogent_driver_last_error().decode()))
+        return {"mean_ms": stats[0], "median_ms": stats[1], "min_ms": stats[2], "max_ms": stats[3], "each_ms": list(each)}
+
+    def time_group(self, group, sizes, c_ptrs, input_ptrs, warmup, iters):
+        self.lib.cogent_driver_time_group.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_int), ctypes.c_int,
+                                                      ctypes.POINTER(ctypes.c_void_p), ctypes.c_int,
+                                                      ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                      ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
+        self.lib.cogent_driver_time_group.restype = ctypes.c_int
+        arr = (ctypes.c_int * len(sizes))(*[int(s) for s in sizes])
+        cb = (ctypes.c_void_p * len(c_ptrs))(*c_ptrs)
+        ib = (ctypes.c_void_p * len(input_ptrs))(*input_ptrs)
+        each = (ctypes.c_float * iters)()
+        stats = (ctypes.c_float * 4)()
+        rc = self.lib.cogent_driver_time_group(group.path.encode(), arr, len(sizes), cb, len(c_ptrs), ib, len(input_ptrs),
+                                               warmup, iters, each, stats)
         if rc:
             raise CogentError("timing failed (%d): %s" % (rc, self.lib.cogent_driver_last_error().decode()))
         return {"mean_ms": stats[0], "median_ms": stats[1], "min_ms": stats[2], "max_ms": stats[3], "each_ms": list(each)}

@@ -1,0 +1,354 @@
+// Fused group of contractions that accumulate into ONE output tensor:
+//
+//     C ±= sum A1*B1;  C ±= sum A2*B2;  ...  (same output index list, any input index orders)
+//
+// -- the reference's "outer group" of expressions with an identical output
+// (cogent/src/algs/bases/tc_gen_inputs.py:113-123), of which the CCSD(T) triples
+// terms are the use: nine contractions into one t3
+// (cogent/drivers/ccsd_t/code_main_sd2_1.c:573-606).  Run one after the other
+// they read and write C nine times; for these 6-D shapes that traffic is the
+// whole cost.  Here a workgroup owns one tile of C for the whole group:
+//
+//   1. the tile is read from global memory once, in C's memory order, into LDS;
+//   2. for every term: both input slices are staged to LDS, contracted on the
+//      matrix cores into zero-initialised accumulators, and the result is added
+//      into the LDS copy.  Which input holds C's fastest index, hence which
+//      side runs along MFMA columns, differs from term to term -- the copy in
+//      LDS is what lets every term use its own lane layout;
+//   3. the tile is written back once.
+//
+// G is the group configuration (C tile, block size), Terms... one Cfg-like
+// struct per term with the members the helpers of tc_kernel.hpp expect.  All
+// tiles are predicated: any extents.
+#pragma once
+#include "tc_launch.hpp"
+
+namespace cogent {
+
+constexpr int TC_MAXTERMS = 16;
+
+// per-term run-time data: the two input pointers and their element strides per index id
+struct TcTermArgs {
+    const void* x;
+    const void* y;
+    int sX[TC_MAXI], sY[TC_MAXI];
+    int enabled;
+};
+
+template <int N>
+struct TcGroupArgs {
+    int ext[TC_MAXI], nblk[TC_MAXI], sC[TC_MAXI];
+    unsigned nblocks;
+    TcTermArgs term[N];
+};
+
+template <class Term> struct TermSlots {
+    static constexpr int X = (Term::BK * Term::BX + Term::NT - 1) / Term::NT;
+    static constexpr int Y = (Term::BK * Term::BY + Term::NT - 1) / Term::NT;
+};
+
+// Geometry of one term for the block's C tile, in the shape the helpers of tc_kernel.hpp take.
+template <class Term>
+struct TermGeom {
+    TcDims d;
+    int rem[Term::NIDX];
+    const typename Term::T* Xb;
+    const typename Term::T* Yb;
+    int nkb;
+};
+
+template <class Term, int NARGS>
+__device__ __forceinline__ void term_setup(TermGeom<Term>& g, const TcGroupArgs<NARGS>& ga, const TcTermArgs& ta, const int* origin)
+{
+    typedef typename Term::T T;
+    int64_t baseX = 0, baseY = 0;
+#pragma unroll
+    for (int i = 0; i < Term::NIDX; i++) {
+        g.d.ext[i] = ga.ext[i]; g.d.nblk[i] = ga.nblk[i]; g.d.sC[i] = ga.sC[i]; g.d.sX[i] = ta.sX[i]; g.d.sY[i] = ta.sY[i];
+        g.rem[i] = ga.ext[i] - origin[i];                     // contracted ids: origin 0
+        baseX += (int64_t)origin[i] * ta.sX[i];
+        baseY += (int64_t)origin[i] * ta.sY[i];
+    }
+    g.nkb = 1;
+#pragma unroll
+    for (int i = 0; i < Term::NK; i++) g.nkb *= (ga.ext[Term::k_id(i)] + Term::k_tile(i) - 1) / Term::k_tile(i);
+    g.Xb = (const T*)ta.x + uniform64(baseX);
+    g.Yb = (const T*)ta.y + uniform64(baseY);
+}
+
+// One term: contract its slices for the block's C tile and add the result into the LDS copy of the tile.
+// (Requesting the next term's first slices while this one is contracted was tried and was 14 % slower.)
+template <class G, class Term, int NARGS>
+__device__ __forceinline__ void group_term(typename G::T* lds_c, typename G::T* lds_ops, const TcGroupArgs<NARGS>& ga,
+                                           const TcTermArgs& ta, const int* origin, int tid)
+{
+    typedef typename G::T T;
+    typedef Mfma<Term::MI> MM;
+    typedef typename MM::Acc Acc;
+    typedef Operand<Term, 0> OX;
+    typedef Operand<Term, 1> OY;
+    constexpr int MT = MM::MT, NREG = MM::NREG, KSTEP = MM::KSTEP, TX = Term::TX, TY = Term::TY, NT = Term::NT;
+    constexpr int LDS_X = lds_elems<OX, Term::BKP>();
+    constexpr int LDS_Y = lds_elems<OY, Term::BKP>();
+    constexpr bool PADDED = (Term::BKP != Term::BK) || (Term::BXP != Term::BX) || (Term::BYP != Term::BY);
+    static_assert(LDS_X + LDS_Y <= G::LDS_OPS, "operand slices exceed the group's LDS share");
+
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wx = wave % Term::WX, wy = wave / Term::WX;
+    T* lds_x = lds_ops;
+    T* lds_y = lds_ops + LDS_X;
+
+    TermGeom<Term> g;
+    term_setup<Term>(g, ga, ta, origin);
+    const TcDims& d = g.d;
+    int* rem = g.rem;
+    const int nkb = g.nkb;
+
+    Acc acc[TY][TX];
+#pragma unroll
+    for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+        for (int tj = 0; tj < TX; tj++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++) acc[ti][tj][r] = (T)0;
+
+    __syncthreads();                       // the previous term is done with the operand region
+    if (PADDED) {
+        for (int i = tid; i < LDS_X + LDS_Y; i += NT) lds_ops[i] = (T)0;
+        __syncthreads();
+    }
+
+    int kbc[Term::NK > 0 ? Term::NK : 1];
+#pragma unroll
+    for (int i = 0; i < Term::NK; i++) kbc[i] = 0;
+    for (int kb = 0; kb < nkb; kb++) {
+        int64_t kx = 0, ky = 0;
+#pragma unroll
+        for (int i = 0; i < Term::NK; i++) {
+            const int id = Term::k_id(i);
+            const int o = kbc[i] * Term::k_tile(i);
+            rem[id] = ga.ext[id] - o;
+            kx += (int64_t)o * ta.sX[id];
+            ky += (int64_t)o * ta.sY[id];
+        }
+        typename Term::T rx[TermSlots<Term>::X], ry[TermSlots<Term>::Y];
+        slice_load<Term, OX, false, false>(rx, g.Xb + uniform64(kx), d, rem, tid);
+        slice_load<Term, OY, false, false>(ry, g.Yb + uniform64(ky), d, rem, tid);
+        if (kb > 0) __syncthreads();       // the previous K block's slices have been consumed
+        slice_store<Term, OX, false>(rx, lds_x, d, tid);
+        slice_store<Term, OY, (Term::SIGN < 0)>(ry, lds_y, d, tid);
+        __syncthreads();
+#pragma unroll
+        for (int k4 = 0; k4 < Term::BKP / KSTEP; k4++) {
+            const int kk = k4 * KSTEP + lane / MT;
+            T a[TY], b[TX];
+#pragma unroll
+            for (int ti = 0; ti < TY; ti++) a[ti] = lds_y[lds_addr<OY>(kk, (wy * TY + ti) * MT + lane % MT)];
+#pragma unroll
+            for (int tj = 0; tj < TX; tj++) b[tj] = lds_x[lds_addr<OX>(kk, (wx * TX + tj) * MT + lane % MT)];
+#pragma unroll
+            for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+                for (int tj = 0; tj < TX; tj++) acc[ti][tj] = MM::mma(a[ti], b[tj], acc[ti][tj]);
+        }
+        // next K block (first composite K index fastest)
+        bool carry = true;
+#pragma unroll
+        for (int i = 0; i < Term::NK; i++) {
+            const int id = Term::k_id(i);
+            const int nb = (ga.ext[id] + Term::k_tile(i) - 1) / Term::k_tile(i);
+            if (carry) { kbc[i]++; carry = false; if (kbc[i] == nb) { kbc[i] = 0; carry = true; } }
+        }
+    }
+
+    // add into the LDS copy of the C tile: every element of the tile belongs to exactly one lane of
+    // this term, and the barriers at the head of the next term order the terms
+#pragma unroll
+    for (int i = 0; i < Term::NK; i++) rem[Term::k_id(i)] = ga.ext[Term::k_id(i)];
+    int cx[TX][1], cy[TY][NREG];
+    c_tile_offsets<Term, false, false, true>(lane, wx, wy, rem, d, cx, cy);
+#pragma unroll
+    for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+        for (int tj = 0; tj < TX; tj++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++)
+                if (cx[tj][0] >= 0 && cy[ti][r] >= 0) lds_c[cx[tj][0] + cy[ti][r]] += acc[ti][tj][r];
+}
+
+template <class G, class... Terms>
+__global__ __launch_bounds__(G::NT)
+void tc_group_kernel(typename G::T* __restrict__ C, const TcGroupArgs<(int)sizeof...(Terms)> ga)
+{
+    typedef typename G::T T;
+    constexpr int NT = G::NT, VOL = G::TILE_VOL;
+    __shared__ __attribute__((aligned(16))) T lds_c[VOL];
+    __shared__ __attribute__((aligned(16))) T lds_ops[G::LDS_OPS];
+    const int tid = threadIdx.x;
+
+    // which C tile: C's indices in C order, fastest first; XCD-contiguous ranges as in the single kernel
+    int origin[G::NIDX];
+#pragma unroll
+    for (int i = 0; i < G::NIDX; i++) origin[i] = 0;
+    int64_t baseC = 0;
+    {
+        const unsigned n = ga.nblocks, xcd = blockIdx.x % 8u, idx = blockIdx.x / 8u;
+        const unsigned q = n / 8u, r = n % 8u;
+        unsigned b = xcd * q + (xcd < r ? xcd : r) + idx;
+#pragma unroll
+        for (int j = 0; j < G::CR; j++) {
+            const int id = G::c_id(j);
+            const unsigned nb = (unsigned)ga.nblk[id];
+            origin[id] = (int)(b % nb) * G::c_tile(j);
+            b /= nb;
+            baseC += (int64_t)origin[id] * ga.sC[id];
+        }
+    }
+    T* __restrict__ Cb = C + uniform64(baseC);
+
+    // element q of the tile in C's memory order: offset in the tensor, inside or outside
+    auto c_element = [&](unsigned q, unsigned& off) -> bool {
+        bool ok = true;
+        off = 0;
+#pragma unroll
+        for (int j = 0; j < G::CR; j++) {
+            const unsigned t = (unsigned)G::c_tile(j);
+            const int c = (int)(q % t);
+            q /= t;
+            const int id = G::c_id(j);
+            off += (unsigned)c * (unsigned)ga.sC[id];
+            ok = ok && (origin[id] + c < ga.ext[id]);
+        }
+        return ok;
+    };
+    constexpr int NEL = (VOL + NT - 1) / NT;
+    {
+        T v[NEL];
+#pragma unroll
+        for (int i = 0; i < NEL; i++) {
+            const unsigned q = (unsigned)(tid + i * NT);
+            unsigned off;
+            v[i] = (T)0;
+            if ((VOL % NT == 0 || q < (unsigned)VOL) && c_element(q, off)) v[i] = Cb[off];
+        }
+#pragma unroll
+        for (int i = 0; i < NEL; i++) {
+            const unsigned q = (unsigned)(tid + i * NT);
+            if (VOL % NT == 0 || q < (unsigned)VOL) lds_c[q] = v[i];
+        }
+    }
+
+    // the terms, in the order of the expression file
+    int t = 0;
+    ((ga.term[t].enabled ? group_term<G, Terms>(lds_c, lds_ops, ga, ga.term[t], origin, tid) : (void)0, t++), ...);
+
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NEL; i++) {
+        const unsigned q = (unsigned)(tid + i * NT);
+        unsigned off;
+        if ((VOL % NT == 0 || q < (unsigned)VOL) && c_element(q, off)) Cb[off] = lds_c[q];
+    }
+}
+
+// Host side.  inputs[] holds the 2 * NTERM input pointers in expression order (A of term 1, B of term 1,
+// A of term 2, ...); enabled[] (may be null: all) says which terms to apply; sizes[] as for tc_run.
+template <class G, class... Terms>
+int tc_group_run(const int* sizes, void* C, const void* const* inputs, const int* enabled, hipStream_t stream)
+{
+    typedef typename G::T T;
+    constexpr int N = (int)sizeof...(Terms);
+    static_assert(N >= 1 && N <= TC_MAXTERMS, "number of fused terms");
+    tc_error_buffer()[0] = 0;
+    for (int i = 0; i < G::NIDX; i++)
+        if (sizes[i] < 0) return tc_fail(TC_ERR_NEGATIVE_EXTENT, "negative extent");
+    for (int i = 0; i < G::NIDX; i++)
+        if (sizes[i] == 0) return TC_OK;
+    if (!C || !inputs) return tc_fail(TC_ERR_NULL_POINTER, "null tensor pointer");
+    for (int i = 0; i < 2 * N; i++)
+        if (!inputs[i] && (!enabled || enabled[i / 2])) return tc_fail(TC_ERR_NULL_POINTER, "null tensor pointer");
+
+    TcGroupArgs<N> ga;
+    memset(&ga, 0, sizeof(ga));
+    const int64_t lim = ((int64_t)1 << 31) - 1;
+    int64_t nC = 1, grid = 1;
+    for (int i = 0; i < G::NIDX; i++) { ga.ext[i] = sizes[i]; ga.nblk[i] = 1; }
+    for (int j = 0; j < G::CR; j++) {
+        const int id = G::c_id(j);
+        ga.sC[id] = (int)nC;
+        nC *= sizes[id];
+        if (nC > lim) return tc_fail(TC_ERR_TOO_LARGE, "a tensor has more than 2^31-1 elements");
+        ga.nblk[id] = (sizes[id] + G::c_tile(j) - 1) / G::c_tile(j);
+        grid *= ga.nblk[id];
+        if (grid > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
+    }
+    ga.nblocks = (unsigned)grid;
+    bool too_large = false;
+    int t = 0;
+    auto fill = [&](auto term) {
+        typedef decltype(term) Term;
+        TcTermArgs& ta = ga.term[t];
+        ta.x = inputs[2 * t + (Term::X_IS_A ? 0 : 1)];
+        ta.y = inputs[2 * t + (Term::X_IS_A ? 1 : 0)];
+        ta.enabled = enabled ? (enabled[t] != 0) : 1;
+        int64_t n = 1;
+        for (int j = 0; j < Term::XR; j++) { ta.sX[Term::xo_id(j)] = (int)n; n *= sizes[Term::xo_id(j)]; if (n > lim) too_large = true; }
+        n = 1;
+        for (int j = 0; j < Term::YR; j++) { ta.sY[Term::yo_id(j)] = (int)n; n *= sizes[Term::yo_id(j)]; if (n > lim) too_large = true; }
+        t++;
+    };
+    (fill(Terms()), ...);
+    if (too_large) return tc_fail(TC_ERR_TOO_LARGE, "a tensor has more than 2^31-1 elements");
+
+    tc_clear_hip_error();
+    hipLaunchKernelGGL((tc_group_kernel<G, Terms...>), dim3((unsigned)grid), dim3(G::NT), 0, stream, (T*)C, ga);
+    return tc_check_launch("fused group kernel launch failed");
+}
+
+// The reference's calling convention for a group: HOST pointers, result copied back.
+template <class G, class... Terms>
+int tc_group_run_host(const int* sizes, void* hC, const void* const* h_inputs)
+{
+    typedef typename G::T T;
+    constexpr int N = (int)sizeof...(Terms);
+    for (int i = 0; i < G::NIDX; i++)
+        if (sizes[i] < 0) return tc_fail(TC_ERR_NEGATIVE_EXTENT, "negative extent");
+    for (int i = 0; i < G::NIDX; i++)
+        if (sizes[i] == 0) return TC_OK;
+    if (!hC || !h_inputs) return tc_fail(TC_ERR_NULL_POINTER, "null tensor pointer");
+    int64_t count[2 * N + 1];
+    {
+        int64_t nC = 1;
+        for (int j = 0; j < G::CR; j++) nC *= sizes[G::c_id(j)];
+        count[2 * N] = nC;
+        int t = 0;
+        auto sz = [&](auto term) {
+            typedef decltype(term) Term;
+            int64_t nx = 1, ny = 1;
+            for (int j = 0; j < Term::XR; j++) nx *= sizes[Term::xo_id(j)];
+            for (int j = 0; j < Term::YR; j++) ny *= sizes[Term::yo_id(j)];
+            count[2 * t + (Term::X_IS_A ? 0 : 1)] = nx;
+            count[2 * t + (Term::X_IS_A ? 1 : 0)] = ny;
+            t++;
+        };
+        (sz(Terms()), ...);
+    }
+    void* dev[2 * N + 1];
+    for (int i = 0; i <= 2 * N; i++) dev[i] = nullptr;
+    int rc = TC_OK;
+    for (int i = 0; i <= 2 * N && rc == TC_OK; i++) {
+        const void* src = (i == 2 * N) ? hC : h_inputs[i];
+        if (!src) { rc = tc_fail(TC_ERR_NULL_POINTER, "null tensor pointer"); break; }
+        if (hipMalloc(&dev[i], count[i] * sizeof(T)) != hipSuccess) rc = tc_fail(TC_ERR_ALLOC, "device allocation failed");
+        else if (hipMemcpy(dev[i], src, count[i] * sizeof(T), hipMemcpyHostToDevice) != hipSuccess) rc = tc_fail(TC_ERR_ALLOC, "host to device copy failed");
+    }
+    if (rc == TC_OK) {
+        rc = tc_group_run<G, Terms...>(sizes, dev[2 * N], (const void* const*)dev, nullptr, 0);
+        if (rc == TC_OK && hipMemcpy(hC, dev[2 * N], count[2 * N] * sizeof(T), hipMemcpyDeviceToHost) != hipSuccess)
+            rc = tc_fail(TC_ERR_LAUNCH, "kernel execution or device to host copy failed");
+    }
+    for (int i = 0; i <= 2 * N; i++) if (dev[i]) (void)hipFree(dev[i]);
+    return rc;
+}
+
+}  // namespace cogent

@@ -55,7 +55,7 @@ int cogent_plan_create(const char* text, const char* dtype, int config_rank, con
     std::vector<Contraction> cs;
     std::string err;
     if (!parse_expression_text(text, cs, err)) return fail(1, err);
-    if (cs.size() != 1) return fail(4, "exactly one expression per plan (fused groups of contractions are not supported)");
+    if (cs.size() != 1) return fail(4, "exactly one expression per plan (several expressions with one output form a fused group: cogent_group_emit)");
     cogent_plan* p = new cogent_plan();
     p->c = cs[0];
     p->t = t;
@@ -94,6 +94,31 @@ int cogent_plan_emit(const cogent_plan* plan, const char* unique_name, const cha
     f << emit_hip_source(plan->c, plan->t, plan->m, unique_name);
     return f.good() ? 0 : fail(5, std::string("cannot write '") + out_path + "'");
 }
+
+static std::string g_group_json;
+
+int cogent_group_emit(const char* text, const char* dtype, const char* tile_spec, const char* unique_name, const char* out_path)
+{
+    if (!text || !dtype || !unique_name) return fail(1, "null argument");
+    DType t;
+    if (!strcmp(dtype, "DOUBLE")) t = DType::F64;
+    else if (!strcmp(dtype, "FLOAT")) t = DType::F32;
+    else return fail(2, std::string("data type must be DOUBLE or FLOAT, got '") + dtype + "'");
+    std::vector<Contraction> cs;
+    std::string err;
+    if (!parse_expression_text(text, cs, err)) return fail(1, err);
+    ArchGfx950 arch;
+    GroupPlan g;
+    if (!plan_group(cs, t, arch, tile_spec ? tile_spec : "", g, err)) return fail(3, err);
+    g_group_json = group_json(g);
+    if (!out_path || !*out_path) return 0;
+    std::ofstream f(out_path);
+    if (!f) return fail(5, std::string("cannot write '") + out_path + "'");
+    f << emit_group_source(g, unique_name);
+    return f.good() ? 0 : fail(5, std::string("cannot write '") + out_path + "'");
+}
+
+const char* cogent_group_last_json(void) { return g_group_json.c_str(); }
 
 const char* cogent_host_last_error(void) { return g_err.c_str(); }
 

@@ -41,11 +41,27 @@ int main(int argc, char** argv)
     if (!f) { fprintf(stderr, "cannot open %s\n", pos[1].c_str()); return 1; }
     std::stringstream ss;
     ss << f.rdbuf();
+    if (name.empty()) name = "tc_" + pos[0];
+    if (out_path.empty()) out_path = "temp__" + pos[0] + ".hip";
+    // several expressions in one file: a fused group (they must share the output), one kernel for all
+    {
+        int n_expr = 0;
+        std::istringstream lines(ss.str());
+        std::string line;
+        while (std::getline(lines, line)) {
+            size_t p = line.find_first_not_of(" \t\r");
+            if (p != std::string::npos && line[p] != '#') n_expr++;
+        }
+        if (n_expr > 1) {
+            int rc = cogent_group_emit(ss.str().c_str(), pos[4].c_str(), spec.empty() ? nullptr : spec.c_str(), name.c_str(), out_path.c_str());
+            if (rc) { fprintf(stderr, "cogent_gen: %s\n", cogent_host_last_error()); return rc; }
+            if (want_json) printf("%s\n", cogent_group_last_json());
+            return 0;
+        }
+    }
     cogent_plan* plan = nullptr;
     int rc = cogent_plan_create(ss.str().c_str(), pos[4].c_str(), atoi(pos[2].c_str()), spec.empty() ? nullptr : spec.c_str(), &plan);
     if (rc) { fprintf(stderr, "cogent_gen: %s\n", cogent_host_last_error()); return rc; }
-    if (name.empty()) name = "tc_" + pos[0];
-    if (out_path.empty()) out_path = "temp__" + pos[0] + ".hip";
     if (want_json) printf("%s\n", cogent_plan_json(plan));
     if (list_k > 0) printf("%s\n", cogent_plan_candidates_json(plan, list_k));
     rc = cogent_plan_emit(plan, name.c_str(), out_path.c_str());

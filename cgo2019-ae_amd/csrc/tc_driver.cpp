@@ -65,6 +65,48 @@ int cogent_driver_time(const char* so_path, const int* sizes, int n_sizes,
     return rc;
 }
 
+// The same measurement for a fused-group object (cogent_run_group): inputs[] holds two pointers per term.
+typedef int (*cogent_run_group_fn)(const int*, int, void*, const void* const*, int, const int*, void*);
+
+int cogent_driver_time_group(const char* so_path, const int* sizes, int n_sizes,
+                             void* const* c_bufs, int n_c_bufs, const void* const* inputs, int n_inputs,
+                             int warmup, int iters, float* ms_each, float* stats)
+{
+    g_err[0] = 0;
+    if (!so_path || !sizes || !c_bufs || !inputs || n_c_bufs < 1 || iters < 1 || warmup < 0) {
+        snprintf(g_err, sizeof g_err, "bad argument");
+        return 1;
+    }
+    void* h = dlopen(so_path, RTLD_NOW | RTLD_LOCAL);
+    if (!h) { snprintf(g_err, sizeof g_err, "dlopen failed: %s", dlerror()); return 2; }
+    cogent_run_group_fn run = (cogent_run_group_fn)dlsym(h, "cogent_run_group");
+    if (!run) { snprintf(g_err, sizeof g_err, "cogent_run_group not exported by %s", so_path); dlclose(h); return 2; }
+    hipStream_t stream = nullptr;
+    std::vector<hipEvent_t> ev(iters + 1);
+    for (auto& e : ev) if (hipEventCreate(&e) != hipSuccess) { snprintf(g_err, sizeof g_err, "hipEventCreate failed"); return 3; }
+    int rc = 0, it = 0;
+    for (int i = 0; i < warmup && !rc; i++, it++) rc = run(sizes, n_sizes, c_bufs[it % n_c_bufs], inputs, n_inputs, nullptr, stream);
+    if (!rc && hipStreamSynchronize(stream) != hipSuccess) rc = 4;
+    if (!rc) (void)hipEventRecord(ev[0], stream);
+    for (int i = 0; i < iters && !rc; i++, it++) {
+        rc = run(sizes, n_sizes, c_bufs[it % n_c_bufs], inputs, n_inputs, nullptr, stream);
+        (void)hipEventRecord(ev[i + 1], stream);
+    }
+    if (hipStreamSynchronize(stream) != hipSuccess && !rc) rc = 4;
+    if (rc) {
+        snprintf(g_err, sizeof g_err, "launch failed with status %d", rc);
+    } else {
+        std::vector<float> ms(iters);
+        double sum = 0;
+        for (int i = 0; i < iters; i++) { (void)hipEventElapsedTime(&ms[i], ev[i], ev[i + 1]); sum += ms[i]; if (ms_each) ms_each[i] = ms[i]; }
+        std::sort(ms.begin(), ms.end());
+        if (stats) { stats[0] = (float)(sum / iters); stats[1] = ms[iters / 2]; stats[2] = ms.front(); stats[3] = ms.back(); }
+    }
+    for (auto& e : ev) (void)hipEventDestroy(e);
+    dlclose(h);
+    return rc;
+}
+
 // Same measurement for a plain device-to-device copy of `bytes` bytes done by a
 // grid-stride kernel: the yardstick the counter readings and the HBM fractions
 // are scaled against.

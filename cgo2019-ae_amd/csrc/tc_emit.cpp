@@ -39,19 +39,12 @@ static std::string c_escape(const std::string& s)
     return o;
 }
 
-std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, const std::string& unique_name)
+// The members every kernel helper expects of a configuration struct (the whole of `Cfg` of a single
+// expression; one `TermN` per contraction of a fused group).
+void emit_cfg_members(std::ostringstream& o, const Contraction& c, DType t, const Mapping& m)
 {
-    std::ostringstream o;
     const char* T = t == DType::F64 ? "double" : "float";
-    // the inputs in the memory order the kernel reads them in (tile order for a repacked input)
     const std::vector<int> xop = operand_order(c, m, true), yop = operand_order(c, m, false);
-
-    o << "// Emitted by cogent-mi355 for gfx950.  Do not edit: regenerate from the expression.\n";
-    o << "//   " << c.text << "\n";
-    o << "//   element type " << T << ", mapping " << m.spec() << "\n";
-    o << "#include \"tc_launch.hpp\"\n\n";
-    o << "namespace {\n";
-    o << "struct Cfg {\n";
     o << "    typedef " << T << " T;\n";
     o << "    static constexpr int NIDX = " << c.n_idx() << ", SIGN = " << c.sign << ";\n";
     o << "    static constexpr bool X_IS_A = " << (m.x_is_a ? "true" : "false") << ";\n";
@@ -107,6 +100,22 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
     o << "    static constexpr int WX = " << m.WX << ", WY = " << m.WY << ", TX = " << m.TX << ", TY = " << m.TY << ", NT = " << 64 * m.WX * m.WY << ";\n";
     o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ", RPX = " << m.RPX << ", RPY = " << m.RPY << ", CLDS = " << m.CLDS << ";\n";
     o << "    static constexpr int LAYX = " << m.layx << ", LDX = " << m.ldx << ", LAYY = " << m.layy << ", LDY = " << m.ldy << ";\n";
+}
+
+std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, const std::string& unique_name)
+{
+    std::ostringstream o;
+    const char* T = t == DType::F64 ? "double" : "float";
+    // the inputs in the memory order the kernel reads them in (tile order for a repacked input)
+    const std::vector<int> xop = operand_order(c, m, true), yop = operand_order(c, m, false);
+
+    o << "// Emitted by cogent-mi355 for gfx950.  Do not edit: regenerate from the expression.\n";
+    o << "//   " << c.text << "\n";
+    o << "//   element type " << T << ", mapping " << m.spec() << "\n";
+    o << "#include \"tc_launch.hpp\"\n\n";
+    o << "namespace {\n";
+    o << "struct Cfg {\n";
+    emit_cfg_members(o, c, t, m);
     o << "};\n";
     o << "}  // namespace\n\n";
 

@@ -104,6 +104,23 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m);
 // the tensor's own order, or for a repacked input its externals in tile order followed by the K indices.
 std::vector<int> operand_order(const Contraction& c, const Mapping& m, bool x_side);
 
+void finish_geometry(const Contraction& c, DType t, Mapping& m);      // tile products, padding, LDS leading dimensions
+
+// ---- fused groups (tc_group.cpp): expressions with one output index list, one kernel
+struct GroupPlan {
+    std::vector<Contraction> terms;
+    DType t = DType::F64;
+    std::vector<int> c_tile;          // tile per output index, in output order
+    std::vector<Mapping> maps;        // per term: roles and tiles derived from c_tile
+    int NW = 4;                       // wavefronts per workgroup
+    int vol = 0, lds_ops = 0;         // elements of the C tile; elements of the largest pair of operand slices
+};
+// spec: empty (search) or "ct=<tile>,<tile>,..." (one per output index)
+bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& arch, const std::string& spec,
+                GroupPlan& g, std::string& err);
+std::string group_json(const GroupPlan& g);
+std::string emit_group_source(const GroupPlan& g, const std::string& unique_name);
+
 // ---- emitter (tc_emit.cpp)
 std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, const std::string& unique_name);
 

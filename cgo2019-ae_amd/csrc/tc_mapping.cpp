@@ -153,7 +153,7 @@ static int lds_ld(int lay, int bep, int bkp, DType t, int mi)
 
 static int fvi(const std::vector<int>& idx) { return idx.empty() ? -1 : idx[0]; }
 
-static void finish_geometry(const Contraction& c, DType t, Mapping& m)
+void finish_geometry(const Contraction& c, DType t, Mapping& m)
 {
     const MiInfo mi = mi_info(m.MI);
     m.BX = 1; for (int v : m.x_tiles) m.BX *= v;

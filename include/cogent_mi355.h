@@ -64,6 +64,30 @@ long long cogent_plan_bytes(const cogent_plan* plan, const int* sizes);
 int cogent_plan_emit(const cogent_plan* plan, const char* unique_name, const char* out_path);
 const char* cogent_host_last_error(void);
 
+/* ---- fused groups ------------------------------------------------------------------------------
+ * Entry points of an object emitted for a group of N expressions (kernels/tc_group.hpp), replacing the
+ * reference's fused interface (cogent/src/codes/kernels/tc_interface.py:1444-1516 with N input pairs):
+ *
+ *   int sd_t_d2_fusion_(int size_<idx>..., T* out, T* a_1, T* b_1, ..., T* a_N, T* b_N,
+ *                       int cond_kernel_1, ..., int cond_kernel_N, int opt_register_transpose);
+ *   int sd_t_d2_fusion_host_(same parameters, HOST pointers);
+ *   int cogent_run_group(const int* sizes, int n_sizes, void* C, const void* const* inputs, int n_inputs,
+ *                        const int* enabled, void* stream);      inputs[] = a_1, b_1, a_2, ...; enabled may be NULL
+ *   int cogent_num_terms(void);   plus cogent_num_indices / cogent_last_error / cogent_expression / cogent_info
+ *
+ * out <- out (+|-) sum a_1*b_1 (+|-) sum a_2*b_2 ...; a term whose cond_kernel flag is 0 is left out.
+ * Same status codes as the single-expression entry points. */
+
+/* Fused group: `text` holds two or more expressions with the same output tensor, output index list,
+ * summed indices and sizes (the reference's outer group, cogent/src/algs/bases/tc_gen_inputs.py:113-123;
+ * the CCSD(T) terms of cogent/drivers/ccsd_t/code_main_sd2_1.c:573-606).  Plans one tile of the output
+ * for the whole group (tile_spec NULL/"" = search, or "ct=<tile>,..." one per output index) and, when
+ * out_path is given, writes ONE translation unit whose kernel keeps the output tile on chip across the
+ * terms.  Returns 0; 1 parse error; 2 data type; 3 no admissible tile / expressions do not form a group;
+ * 5 file.  cogent_group_last_json() describes the plan of the last successful call. */
+int cogent_group_emit(const char* text, const char* dtype, const char* tile_spec, const char* unique_name, const char* out_path);
+const char* cogent_group_last_json(void);
+
 /* Seeded inputs: element i = 2 * u_i - 1 with u_i in [0,1) taken from the top
  * bits of splitmix64(seed + (i + 1) * 0x9E3779B97F4A7C15), so the fill does not
  * depend on the tensor's shape.  (The reference fills with unseeded
