@@ -21,8 +21,8 @@ def declared_functions():
 def test_header_declarations_are_exported():
     names = declared_functions()
     host = ctypes.CDLL(os.path.join(PKG, "lib", "libcogent_mi355.so"))
-    host_names = [n for n in names if n.startswith(("cogent_plan_", "cogent_fill_", "cogent_host_"))]
-    assert len(host_names) >= 10
+    host_names = [n for n in names if n.startswith(("cogent_plan_", "cogent_fill_", "cogent_host_", "cogent_group_"))]
+    assert len(host_names) >= 12
     for n in host_names:
         assert hasattr(host, n), n
     per_expression = [n for n in names if n not in host_names]
@@ -44,7 +44,7 @@ def test_every_expression_object_exports_the_entry_points():
 def test_driver_library_exports():
     out = subprocess.run(["nm", "-D", "--defined-only", os.path.join(PKG, "lib", "libcogent_driver.so")],
                          stdout=subprocess.PIPE, text=True, check=True).stdout
-    for s in ("cogent_driver_time", "cogent_driver_time_copy", "cogent_driver_last_error"):
+    for s in ("cogent_driver_time", "cogent_driver_time_group", "cogent_driver_time_copy", "cogent_driver_last_error"):
         assert s in out
 
 

@@ -8,7 +8,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 EXPR_DIR = os.path.join(ROOT, "cgo2019-ae_amd", "expressions")
-FILES = sorted(glob.glob(os.path.join(EXPR_DIR, "*.in")))
+FILES = sorted(p for p in glob.glob(os.path.join(EXPR_DIR, "*.in")) if not os.path.basename(p).startswith("fused_"))   # groups: tests/test_groups.py
 MT = {"v_mfma_f64_16x16x4_f64": (16, 4), "v_mfma_f32_16x16x4_f32": (16, 4), "v_mfma_f32_32x32x2_f32": (32, 2)}
 
 
