@@ -496,7 +496,7 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
                         // few output tiles and a long K loop: also try splitting K over 2, 4, 8 workgroups
                         const long long tiles = m.n_blocks;
                         const int ksteps = m.steps_main_loop;
-                        for (int sk = 2; sk <= 8 && tiles < 8LL * arch.n_cu && ksteps >= 8 * sk; sk *= 2) {
+                        for (int sk = 2; sk <= 64 && tiles * (sk / 2) < 4LL * arch.n_cu && ksteps >= 8 * sk; sk *= 2) {
                             Mapping ms = m;
                             ms.SK = sk;
                             cost_model(c, t, arch, ms);
