@@ -77,6 +77,7 @@ template <> struct Mfma<2> {   // v_mfma_f32_32x32x2_f32
 template <class Cfg, int SIDE> struct Operand;
 template <class Cfg> struct Operand<Cfg, 0> {
     static constexpr int R = Cfg::XR, LAY = Cfg::LAYX, LD = Cfg::LDX, BE = Cfg::BX, BEP = Cfg::BXP;
+    static constexpr bool NTL = (Cfg::NTO & 1) != 0;      // this input is read once: non-temporal loads
     __device__ static __forceinline__ constexpr int id(int j)   { return Cfg::xo_id(j); }
     __device__ static __forceinline__ constexpr int tile(int j) { return Cfg::xo_tile(j); }
     __device__ static __forceinline__ constexpr int isk(int j)  { return Cfg::xo_isk(j); }
@@ -85,6 +86,7 @@ template <class Cfg> struct Operand<Cfg, 0> {
 };
 template <class Cfg> struct Operand<Cfg, 1> {
     static constexpr int R = Cfg::YR, LAY = Cfg::LAYY, LD = Cfg::LDY, BE = Cfg::BY, BEP = Cfg::BYP;
+    static constexpr bool NTL = (Cfg::NTO & 2) != 0;
     __device__ static __forceinline__ constexpr int id(int j)   { return Cfg::yo_id(j); }
     __device__ static __forceinline__ constexpr int tile(int j) { return Cfg::yo_tile(j); }
     __device__ static __forceinline__ constexpr int isk(int j)  { return Cfg::yo_isk(j); }
@@ -156,7 +158,7 @@ __device__ __forceinline__ void slice_load(typename Cfg::T (&reg)[SLOTS], const 
         unsigned goff; int loff; bool valid;
         slice_element<Op, EXT_FULL, INT_FULL>(q, d, rem, goff, loff, valid);
         T v = (T)0;
-        if ((E % Cfg::NT == 0 || q < E) && valid) v = *(const T*)((const char*)src + goff * (unsigned)sizeof(T));
+        if ((E % Cfg::NT == 0 || q < E) && valid) v = c_load<Op::NTL>((const T*)((const char*)src + goff * (unsigned)sizeof(T)));
         reg[s] = v;
     }
 }

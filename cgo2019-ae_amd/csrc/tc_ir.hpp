@@ -75,6 +75,7 @@ struct Mapping {
     int RPX = 0, RPY = 0;                     // 1 (mapping spec rx=/ry= only): that input is first copied into tile order, see operand_order()
     int CLDS = 0;                             // 1: full C tiles pass through LDS in C's memory order (16-byte, whole-line global accesses)
     int clds_forced = -1;
+    int NTO = 0, nto_forced = -1;             // non-temporal input loads: bit 0 X side, bit 1 Y side (an input every element of which is read once)
     int SK = 1;                               // split-K factor: SK workgroups per output tile, atomic accumulate
     int layx = 0, ldx = 0, layy = 0, ldy = 0; // LDS layout per operand
     // model outputs

@@ -69,6 +69,7 @@ std::string Mapping::spec() const
     if (swap_forced >= 0) o << ";sw=" << swap_forced;
     if (pd_forced >= 1) o << ";pd=" << pd_forced;
     if (clds_forced >= 0) o << ";cl=" << clds_forced;
+    if (nto_forced >= 0) o << ";no=" << nto_forced;
     if (RPX) o << ";rx=1";
     if (RPY) o << ";ry=1";
     return o.str();
@@ -243,6 +244,10 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     for (size_t i = 0; i < m.y_ids.size(); i++) nblocks *= ceil_div(c.indices[m.y_ids[i]].rep_size, m.y_tiles[i]);
     long long nkb = 1;
     for (size_t i = 0; i < m.k_ids.size(); i++) nkb *= ceil_div(c.indices[m.k_ids[i]].rep_size, m.k_tiles[i]);
+    // non-temporal input loads (mapping spec no= only: bit 0 X side, bit 1 Y side), meant for an input
+    // every element of which is read once.  Measured: config 1's 134 MB input, read once in 128-byte
+    // pieces, got 6 % slower with the hint; TCCG-15 6 % faster.  Never chosen automatically.
+    m.NTO = m.nto_forced >= 0 ? m.nto_forced : 0;
     // split K: SK workgroups per tile, each a share of the K blocks, accumulated with atomics
     const int sk = (nkb > 1) ? std::max(1, m.SK) : 1;
     const double c_passes = sk > 1 ? (double)sk : 1.0;
@@ -571,6 +576,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "sw") m.swap_forced = atoi(val.c_str()) ? 1 : 0;
         else if (key == "pd") m.pd_forced = std::max(1, std::min(8, atoi(val.c_str())));
         else if (key == "cl") m.clds_forced = atoi(val.c_str()) ? 1 : 0;
+        else if (key == "no") m.nto_forced = std::max(0, std::min(3, atoi(val.c_str())));
         else if (key == "rx") m.RPX = atoi(val.c_str()) ? 1 : 0;
         else if (key == "ry") m.RPY = atoi(val.c_str()) ? 1 : 0;
         else if (key == "lx") lx = atoi(val.c_str());
@@ -604,7 +610,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

@@ -64,12 +64,20 @@ def test_group_tile_spec_and_rejections(tmp_path):
     assert rc == 3 and "must share the output" in err
 
 
-def test_group_object_exports_the_fused_entry_points():
-    so = os.path.join(PKG, "lib", "fused_sd2_f64.so")
+@pytest.mark.parametrize("name", ["fused_sd2_f64", "fused_sd1_f32"])
+def test_group_object_exports_the_fused_entry_points(name):
+    so = os.path.join(PKG, "lib", name + ".so")
     out = subprocess.run(["nm", "-D", "--defined-only", so], stdout=subprocess.PIPE, text=True, check=True).stdout
-    for sym in ("sd_t_d2_fusion_", "sd_t_d2_fusion_host_", "cogent_run_group", "cogent_fused_sd2_f64_run_group",
+    for sym in ("sd_t_d2_fusion_", "sd_t_d2_fusion_host_", "cogent_run_group", "cogent_%s_run_group" % name,
                 "cogent_num_indices", "cogent_num_terms", "cogent_last_error", "cogent_expression", "cogent_info"):
         assert (" T " + sym + "\n") in out, sym
+
+
+def test_fp32_group_plan():
+    rc, j = plan_json(os.path.join(PKG, "expressions", "fused_sd1_f32.in"), dtype="FLOAT")
+    assert rc == 0 and j["dtype"] == "f32" and j["n_terms"] == 9 and j["sum_idx"] == ["h7"]
+    assert int(np.prod(j["c_tile"])) * 4 <= 32768
+    assert all(t["mapping"]["mfma"] == "v_mfma_f32_16x16x4_f32" for t in j["terms"])
 
 
 def expected(terms, sizes, C, inputs, oracle, enabled=None):
@@ -80,17 +88,21 @@ def expected(terms, sizes, C, inputs, oracle, enabled=None):
     return want
 
 
+TOL = {"f64": 1e-12, "f32": 1e-5}
+
+
 def run_group(g, terms, sizes, tools, oracle, enabled=None, via="entry"):
     import torch
     from gpu_common import DeviceTensor
+    dt = np.float64 if g.dtype == "f64" else np.float32
     rng_seed = 10
     inputs = []
     for expr in terms:
         _, nA, nB = helpers.tensor_sizes(expr, sizes)
-        inputs.append(tools.fill_uniform(np.empty(nA, np.float64), rng_seed)); rng_seed += 1
-        inputs.append(tools.fill_uniform(np.empty(nB, np.float64), rng_seed)); rng_seed += 1
+        inputs.append(tools.fill_uniform(np.empty(nA, dt), rng_seed)); rng_seed += 1
+        inputs.append(tools.fill_uniform(np.empty(nB, dt), rng_seed)); rng_seed += 1
     nC = helpers.tensor_sizes(terms[0], sizes)[0]
-    C = tools.fill_uniform(np.empty(nC, np.float64), 3)
+    C = tools.fill_uniform(np.empty(nC, dt), 3)
     dC = DeviceTensor(C)
     dI = [DeviceTensor(a) for a in inputs]
     ptrs = [d.ptr for d in dI]
@@ -104,21 +116,26 @@ def run_group(g, terms, sizes, tools, oracle, enabled=None, via="entry"):
     return dC.host(), expected(terms, sizes, C, inputs, oracle, enabled)
 
 
-@pytest.fixture(scope="module")
-def group():
+def load_group(name):
     import cogent_mi355
-    g = cogent_mi355.Group("fused_sd2_f64")
+    g = cogent_mi355.Group(name)
     return g, [helpers.parse_expression(t) for t in g.expressions]
 
 
+@pytest.fixture(scope="module")
+def group():
+    return load_group("fused_sd2_f64")
+
+
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["fused_sd2_f64", "fused_sd1_f32"])
 @pytest.mark.parametrize("sizes", [[5, 3, 7, 6, 2, 9, 4], [16, 4, 4, 2, 2, 2, 16], [17, 5, 6, 3, 4, 3, 19], [1, 1, 1, 1, 1, 1, 1],
-                                   [32, 8, 4, 4, 4, 2, 24]])
-def test_fused_group_matches_the_terms_applied_one_by_one(sizes, group, tools, oracle):
-    g, terms = group
+                                   [32, 8, 4, 4, 4, 2, 24], [16, 16, 16, 16, 8, 8, 16]])
+def test_fused_group_matches_the_terms_applied_one_by_one(name, sizes, tools, oracle):
+    g, terms = load_group(name)
     assert g.n_terms == 9 and g.n == 7
     got, want = run_group(g, terms, sizes, tools, oracle)
-    assert helpers.rel_error(got, want) <= 1e-12
+    assert helpers.rel_error(got, want) <= TOL[g.dtype]
 
 
 @pytest.mark.gpu

@@ -94,6 +94,10 @@ def test_kernel_options_in_a_spec(tools):
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:24,a:2;k=e:12;w=3x1;t=3x3;rx=1;ry=1").info["mapping"]
     assert m["repack"] == [1, 1] and m["lds_layout"] == [0, 0] and "rx=1" in m["spec"] and "ry=1" in m["spec"]
     assert tools.plan(text, "DOUBLE").info["mapping"]["repack"] == [0, 0]      # never chosen automatically
+    # no=: non-temporal loads of an input (bit 0 X side, bit 1 Y side), opt-in
+    m = tools.plan(text, "DOUBLE", mapping_spec=base + ";no=2").info["mapping"]
+    assert m["nontemporal_inputs"] == 2 and "no=2" in m["spec"]
+    assert tools.plan(text, "DOUBLE", mapping_spec=base).info["mapping"]["nontemporal_inputs"] == 0
     # cl=1: the C tile passes through LDS in memory order (opt-in; refused silently when the tile is too large)
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:8,c:8;y=b:24,a:2;k=e:8;w=2x1;t=2x3;cl=1").info["mapping"]
     assert m["c_through_lds"] == 1 and "cl=1" in m["spec"]
