@@ -38,7 +38,7 @@ static std::string c_escape(const std::string& s)
 
 // The mapping of one term for a given tile of C.  Returns false when the term cannot be laid out
 // (accumulators or LDS out of budget).
-static bool term_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const std::vector<int>& c_tile, int NW,
+static bool term_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const std::vector<int>& c_tile, int NW, int k_room,
                          Mapping& m, std::string& err)
 {
     m = Mapping();
@@ -51,8 +51,8 @@ static bool term_mapping(const Contraction& c, DType t, const ArchGfx950& arch, 
         if (pos_in(xop, id) >= 0) { m.x_ids.push_back(id); m.x_tiles.push_back(c_tile[j]); }
         else                      { m.y_ids.push_back(id); m.y_tiles.push_back(c_tile[j]); }
     }
-    // contracted indices in the X input's order, at most 32 deep per K block
-    int room = 32;
+    // contracted indices in the X input's order, at most k_room deep per K block
+    int room = k_room;
     for (int id : xop) {
         if (!c.indices[id].internal) continue;
         const int rep = c.indices[id].rep_size;
@@ -103,7 +103,6 @@ bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& a
     }
     g.terms = cs;
     g.t = t;
-    g.NW = 4;
     const int s = esize(t);
     const int CR = (int)c0.out_idx.size();
     const int vol_max = 32768 / s;
@@ -118,7 +117,7 @@ bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& a
         int lds_ops = 0;
         for (size_t k = 0; k < cs.size(); k++) {
             std::string e;
-            if (!term_mapping(cs[k], t, arch, tile, g.NW, maps[k], e)) { why = "term " + std::to_string(k + 1) + ": " + e; return false; }
+            if (!term_mapping(cs[k], t, arch, tile, g.NW, g.k_room, maps[k], e)) { why = "term " + std::to_string(k + 1) + ": " + e; return false; }
             const Mapping& m = maps[k];
             if (m.lds_bytes > 32768) { why = "term " + std::to_string(k + 1) + ": input slices exceed 32 KB"; return false; }
             lds_ops = std::max(lds_ops, m.lds_bytes);
@@ -146,10 +145,21 @@ bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& a
     };
 
     std::vector<int> tile(CR, 1);
-    if (!spec.empty()) {
-        // ct=<tile>,<tile>,...  one per output index, in output order
-        if (spec.compare(0, 3, "ct=") != 0) { err = "group mapping spec must be ct=<tile>,<tile>,... (one per output index)"; return false; }
-        std::istringstream is(spec.substr(3));
+    std::string ct_spec;
+    {
+        // fields separated by ';': ct=<tile>,<tile>,... (one per output index), kt=<K depth per block>, nw=<wavefronts>
+        std::istringstream fs(spec);
+        std::string field;
+        while (std::getline(fs, field, ';')) {
+            if (field.empty()) continue;
+            if (field.compare(0, 3, "ct=") == 0) ct_spec = field.substr(3);
+            else if (field.compare(0, 3, "kt=") == 0) g.k_room = std::max(4, std::min(64, atoi(field.c_str() + 3)));
+            else if (field.compare(0, 3, "nw=") == 0) g.NW = std::max(1, std::min(8, atoi(field.c_str() + 3)));
+            else { err = "group mapping spec: fields are ct=<tile>,... kt=<n> nw=<n>"; return false; }
+        }
+    }
+    if (!ct_spec.empty()) {
+        std::istringstream is(ct_spec);
         std::string item;
         int j = 0;
         while (std::getline(is, item, ',')) { if (j < CR) tile[j] = atoi(item.c_str()); j++; }
@@ -195,7 +205,7 @@ std::string group_json(const GroupPlan& g)
     for (size_t j = 0; j < g.c_tile.size(); j++) o << (j ? ", " : "") << g.c_tile[j];
     o << "], \"threads\": " << 64 * g.NW << ", \"lds_bytes\": " << (g.vol + g.lds_ops) * esize(g.t) << ", \"spec\": \"ct=";
     for (size_t j = 0; j < g.c_tile.size(); j++) o << (j ? "," : "") << g.c_tile[j];
-    o << "\", \"terms\": [";
+    o << ";kt=" << g.k_room << ";nw=" << g.NW << "\", \"terms\": [";
     for (size_t k = 0; k < g.terms.size(); k++)
         o << (k ? ", " : "") << "{\"text\": \"" << c_escape(g.terms[k].text) << "\", \"mapping\": " << mapping_json(g.terms[k], g.t, g.maps[k]) << "}";
     o << "]}";

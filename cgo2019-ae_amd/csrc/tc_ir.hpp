@@ -114,9 +114,10 @@ struct GroupPlan {
     std::vector<int> c_tile;          // tile per output index, in output order
     std::vector<Mapping> maps;        // per term: roles and tiles derived from c_tile
     int NW = 4;                       // wavefronts per workgroup
+    int k_room = 32;                  // contracted depth per K block
     int vol = 0, lds_ops = 0;         // elements of the C tile; elements of the largest pair of operand slices
 };
-// spec: empty (search) or "ct=<tile>,<tile>,..." (one per output index)
+// spec: empty (search) or fields "ct=<tile>,<tile>,..." (one per output index), "kt=<K depth>", "nw=<wavefronts>" joined by ';'
 bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& arch, const std::string& spec,
                 GroupPlan& g, std::string& err);
 std::string group_json(const GroupPlan& g);

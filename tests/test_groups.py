@@ -52,7 +52,11 @@ def test_group_plan_shares_one_tile_and_gives_each_term_its_own_roles():
 
 def test_group_tile_spec_and_rejections(tmp_path):
     rc, j = plan_json(FUSED, spec="ct=16,2,2,4,2,2")
-    assert rc == 0 and j["c_tile"] == [16, 2, 2, 4, 2, 2] and j["spec"] == "ct=16,2,2,4,2,2"
+    assert rc == 0 and j["c_tile"] == [16, 2, 2, 4, 2, 2] and j["spec"] == "ct=16,2,2,4,2,2;kt=32;nw=4"
+    rc, j = plan_json(FUSED, spec="ct=16,4,4,2,2,2;kt=8;nw=8")                 # K depth per block, wavefronts per workgroup
+    assert rc == 0 and j["threads"] == 512 and all(t["mapping"]["block_tile"][2] == 8 for t in j["terms"])
+    rc, err = plan_json(FUSED, spec="tile=3")
+    assert rc == 3 and "fields are" in err
     rc, err = plan_json(FUSED, spec="ct=16,16,16,16,1,1")              # 64 K elements of C: does not fit
     assert rc == 3 and "does not fit" in err
     rc, err = plan_json(FUSED, spec="ct=16,2,2")
