@@ -16,8 +16,8 @@ from gpu_common import make_inputs, run_entry
 pytestmark = pytest.mark.gpu
 
 TOL = {"f64": 1e-12, "f32": 1e-5}
-SMALL = [3, 4, 5, 2, 6, 3, 4]
-ODD = [17, 5, 3, 9, 2, 7, 19]
+SMALL = [3, 4, 5, 2, 6, 3, 4, 2, 3, 5, 2, 3]
+ODD = [17, 5, 3, 9, 2, 7, 19, 3, 6, 5, 4, 2]
 
 
 def _pkg():
@@ -105,6 +105,16 @@ def test_odd_extents_mixed_full_and_partial(name, tools, oracle):
     int_partial = [min(f, 16) for f in full[:n_out]] + cap(odd[n_out:])
     check(name, ext_partial, tools, oracle)
     check(name, int_partial, tools, oracle)
+
+
+@pytest.mark.parametrize("name", [n for n in all_names() if n.startswith("rand_")])
+def test_random_expressions_at_their_own_and_at_odd_sizes(name, tools, oracle):
+    """The seeded random expressions (expressions/make_random.py): at the sizes they were mapped for, and
+    at odd sizes that divide none of their tiles."""
+    pkg = _pkg()
+    n = pkg.Expression(name).n
+    check(name, pkg.manifest_entry(name)["bench_sizes"], tools, oracle)
+    check(name, ODD[:n], tools, oracle)
 
 
 @pytest.mark.parametrize("name", ["cfg1_f64", "cfg3_f64", "cfg4_f32", "cfg5_3_f64"])
