@@ -82,3 +82,34 @@ def test_two_calls_accumulate(tools, oracle):
     torch.cuda.synchronize()
     want = oracle.contract(expr, sizes, oracle.contract(expr, sizes, C.copy(), A, B), A, B)
     assert helpers.rel_error(dC.host(), want) <= 1e-12
+
+
+@pytest.mark.gpu
+def test_entry_point_inside_a_captured_graph(tools, oracle):
+    """cogent_run on a caller's stream allocates nothing and does not synchronise, so a sequence of calls can be
+    captured into a HIP graph and replayed: three replays, each checked against the eager result."""
+    import torch
+    import cogent_mi355
+    ex = cogent_mi355.Expression("cfg5_1_f64")
+    expr = helpers.parse_expression(cogent_mi355.expression_text("cfg5_1_f64"))
+    sizes = [8, 6, 5, 7, 4, 6, 9]
+    C, A, B = make_inputs(tools, expr, sizes, np.float64)
+    want1 = oracle.contract(expr, sizes, C.copy(), A, B)
+    want2 = oracle.contract(expr, sizes, want1.copy(), A, B)          # two launches per replay
+    dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    dC = torch.from_numpy(C).cuda()
+    dC0 = dC.clone()
+    s = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    print("[gpu] graph capture of cfg5_1_f64 sizes=%s" % sizes, flush=True)
+    with torch.cuda.graph(g, stream=s):
+        st = torch.cuda.current_stream().cuda_stream
+        assert ex.run(sizes, dC.data_ptr(), dA.data_ptr(), dB.data_ptr(), st, 0) == 0
+        assert ex.run(sizes, dC.data_ptr(), dA.data_ptr(), dB.data_ptr(), st, 0) == 0
+    for replay in range(3):
+        dC.copy_(dC0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = dC.cpu().numpy()
+        assert helpers.rel_error(got, want2) <= 1e-12, "replay %d" % replay
