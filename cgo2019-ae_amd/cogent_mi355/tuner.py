@@ -64,7 +64,16 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     gen = os.path.join(b.BIN, "cogent_gen")
     src = os.path.join(b.EXPR, entry["file"])
     listing = b.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", os.devnull, "--list", str(max(4 * top_k, 40))])
-    specs = list(extra_specs) + [c["spec"] for c in distinct_candidates(json.loads(listing), top_k)]
+    cands = distinct_candidates(json.loads(listing), top_k)
+    specs = list(extra_specs) + [c["spec"] for c in cands]
+    # long K loops: the three best tilings also with two K blocks in flight, with and without asking the
+    # register allocator to keep three wavefronts per SIMD (the deeper prefetch costs registers)
+    deep = [c["spec"] for c in cands if c["model"]["k_steps"] >= 8][:3]
+    if cands and cands[0]["model"]["k_steps"] >= 8:
+        deep = [s for s in extra_specs if "pd=" not in s] + deep      # the mappings handed in defend their place in both forms
+    for sp in deep:
+        base = ";".join(f for f in sp.split(";") if not f.startswith("mw="))
+        specs += [base + ";pd=2", base + ";pd=2;mw=3"]
     if entry.get("map") and entry["map"] not in specs:
         specs.insert(0, entry["map"])                      # the pinned mapping defends its place
     out = os.path.join(out_root, name)
