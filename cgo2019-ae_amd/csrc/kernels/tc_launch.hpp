@@ -12,6 +12,7 @@
 #include <stdio.h>
 #include <string.h>
 #include "tc_kernel.hpp"
+#include "tc_stream.hpp"
 
 namespace cogent {
 
@@ -44,6 +45,10 @@ inline int tc_check_launch(const char* what)
 
 enum TcVariant { TC_VARIANT_AUTO = 0, TC_VARIANT_PLAIN = 1, TC_VARIANT_TILED = 2 };
 
+// Which kernel the last call of this thread launched (0: none yet, or the call returned before a launch).
+enum TcKernelKind { TC_KERNEL_NONE = 0, TC_KERNEL_PLAIN = 1, TC_KERNEL_TILED = 2, TC_KERNEL_STREAM = 3 };
+inline int& tc_last_kernel() { static thread_local int kind = TC_KERNEL_NONE; return kind; }
+
 template <class Cfg, bool ONE_KB, bool SWP>
 inline void tc_launch_full_partial(bool ext_full, bool int_full, dim3 g, dim3 b, hipStream_t stream,
                                    typename Cfg::T* c, const typename Cfg::T* x, const typename Cfg::T* y, const TcDims& d)
@@ -69,6 +74,56 @@ inline void tc_launch_variant(bool one_kb, bool ext_full, bool int_full, bool sw
     else        tc_launch_full_partial<Cfg, false, false>(ext_full, int_full, g, b, stream, c, x, y, d);
 }
 
+// The panel-resident streaming kernel, when the object carries one (Cfg::STREAM = its K-block count)
+// and this call has full tiles and exactly that many K blocks.  Returns false when the call has to
+// go to the per-tile kernel instead.  The grid is sized so that all workgroups are resident at once:
+// every X-side tile gets as many runs of consecutive Y-side tiles as fill the CUs about once.
+template <class Cfg>
+inline bool tc_stream_launch(bool ext_full, bool int_full, int64_t nkb, bool swp, hipStream_t stream,
+                             typename Cfg::T* c, const typename Cfg::T* x, const typename Cfg::T* y, const TcDims& d)
+{
+    if constexpr (Cfg::STREAM > 0) {
+        typedef typename Cfg::T T;
+        if (!ext_full || !int_full || nkb != Cfg::STREAM) return false;
+        constexpr size_t lds_bytes = sizeof(T) * ((size_t)Cfg::STREAM * lds_elems<Operand<Cfg, 0>, Cfg::BKP>() + 2 * (size_t)lds_elems<Operand<Cfg, 1>, Cfg::BKP>());
+        static_assert(lds_bytes <= 160 * 1024, "X panel does not fit the LDS");
+        static int n_cu = 0;
+        if (n_cu == 0) {
+            int dev = 0, v = 0;
+            if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 1) {
+                (void)hipGetLastError();
+                return false;
+            }
+            n_cu = v;
+        }
+        const void* fn = swp ? (const void*)&tc_stream_kernel<Cfg, Cfg::SWAP != 0> : (const void*)&tc_stream_kernel<Cfg, false>;
+        static bool configured[2] = {false, false};
+        if (!configured[swp ? 1 : 0]) {
+            if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) {
+                (void)hipGetLastError();
+                return false;
+            }
+            configured[swp ? 1 : 0] = true;
+        }
+        const int by_lds = (int)((160 * 1024) / lds_bytes), by_regs = (Cfg::SMW * 4 * 64) / Cfg::NT;
+        const int64_t slots = (int64_t)n_cu * (by_lds < by_regs ? by_lds : (by_regs < 1 ? 1 : by_regs));
+        TcStreamDims s;
+        s.nyt = d.nblocks / d.nxt;
+        int64_t runs = slots / d.nxt;                        // runs per X tile: as many as keep the whole grid resident at once
+        if (runs < 1) runs = 1;
+        if (runs > s.nyt) runs = s.nyt;
+        s.run = (unsigned)((s.nyt + runs - 1) / runs);
+        s.nruns = (s.nyt + s.run - 1) / s.run;
+        const dim3 g(d.nxt * s.nruns), b(Cfg::NT);
+        if (swp) hipLaunchKernelGGL((tc_stream_kernel<Cfg, Cfg::SWAP != 0>), g, b, lds_bytes, stream, c, x, y, d, s);
+        else     hipLaunchKernelGGL((tc_stream_kernel<Cfg, false>), g, b, lds_bytes, stream, c, x, y, d, s);
+        return true;
+    } else {
+        (void)ext_full; (void)int_full; (void)nkb; (void)swp; (void)stream; (void)c; (void)x; (void)y; (void)d;
+        return false;
+    }
+}
+
 // sizes[] holds one extent per index id: output indices in output order, then
 // the contracted indices in sum() order -- the order of the entry point's
 // `int size_*` parameters (cogent/src/codes/kernels/tc_interface.py:1459-1492).
@@ -77,6 +132,7 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
 {
     typedef typename Cfg::T T;
     tc_error_buffer()[0] = 0;
+    tc_last_kernel() = TC_KERNEL_NONE;
     if (variant < 0 || variant > 2) return tc_fail(TC_ERR_BAD_VARIANT, "unknown kernel variant");
     for (int i = 0; i < Cfg::NIDX; i++)
         if (sizes[i] < 0) return tc_fail(TC_ERR_NEGATIVE_EXTENT, "negative extent");
@@ -116,6 +172,7 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
         tc_clear_hip_error();
         hipLaunchKernelGGL(tc_plain_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream,
                            (T*)C, (const T*)A, (const T*)B, p);
+        tc_last_kernel() = TC_KERNEL_PLAIN;
         return tc_check_launch("plain kernel launch failed");
     }
 
@@ -199,7 +256,12 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     const dim3 g((unsigned)grid), b(Cfg::NT);
     // swapped MFMA roles with 128-bit C accesses: fp32 only, fastest extent a multiple of 4, C 16-byte aligned
     const bool swp = Cfg::SWAP && (sizes[Cfg::c_id(0)] % 4 == 0) && (((uintptr_t)C & 15) == 0);
-    tc_launch_variant<Cfg>(nkb == 1, ext_full, int_full, swp, g, b, stream, c, x, y, d);
+    if (variant == TC_VARIANT_AUTO && tc_stream_launch<Cfg>(ext_full, int_full, nkb, swp, stream, c, x, y, d)) {
+        tc_last_kernel() = TC_KERNEL_STREAM;
+    } else {
+        tc_launch_variant<Cfg>(nkb == 1, ext_full, int_full, swp, g, b, stream, c, x, y, d);
+        tc_last_kernel() = TC_KERNEL_TILED;
+    }
     const int rc = tc_check_launch("tiled kernel launch failed");
     if (ws && hipFreeAsync(ws, stream) != hipSuccess) { (void)hipGetLastError(); if (rc == TC_OK) return tc_fail(TC_ERR_ALLOC, "stream-ordered free of the repack buffer failed"); }
     return rc;

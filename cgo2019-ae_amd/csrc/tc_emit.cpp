@@ -99,6 +99,7 @@ void emit_cfg_members(std::ostringstream& o, const Contraction& c, DType t, cons
     operand("Y", yop, m.y_ids, m.y_tiles);
     o << "    static constexpr int WX = " << m.WX << ", WY = " << m.WY << ", TX = " << m.TX << ", TY = " << m.TY << ", NT = " << 64 * m.WX * m.WY << ";\n";
     o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ", RPX = " << m.RPX << ", RPY = " << m.RPY << ", CLDS = " << m.CLDS << ", NTO = " << m.NTO << ";\n";
+    o << "    static constexpr int STREAM = " << m.STREAM << ", SPD = " << m.SPD << ", SMW = " << m.SMW << ";\n";
     o << "    static constexpr int LAYX = " << m.layx << ", LDX = " << m.ldx << ", LAYY = " << m.layy << ", LDY = " << m.ldy << ";\n";
 }
 
@@ -149,6 +150,7 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
     o << "    return cogent_run(sizes, n_sizes, C, A, B, stream, variant);\n}\n\n";
     o << "int cogent_num_indices(void) { return Cfg::NIDX; }\n";
     o << "const char* cogent_last_error(void) { return cogent::tc_error_buffer(); }\n";
+    o << "int cogent_last_kernel(void) { return cogent::tc_last_kernel(); }\n";
     o << "const char* cogent_expression(void) { return \"" << c_escape(c.text) << "\"; }\n";
     o << "const char* cogent_info(void) { return \"" << c_escape(mapping_json(c, t, m)) << "\"; }\n";
     o << "\n}  // extern \"C\"\n";

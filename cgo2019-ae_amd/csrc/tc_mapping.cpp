@@ -70,6 +70,7 @@ std::string Mapping::spec() const
     if (pd_forced >= 1) o << ";pd=" << pd_forced;
     if (clds_forced >= 0) o << ";cl=" << clds_forced;
     if (nto_forced >= 0) o << ";no=" << nto_forced;
+    if (st_forced > 0) o << ";st=" << st_forced;
     if (RPX) o << ";rx=1";
     if (RPY) o << ";ry=1";
     return o.str();
@@ -366,8 +367,15 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const double simd_busy = std::min(waves_simd / std::ceil(waves_simd), per_block);
     const double n_mfma = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * (m.BXP / mi.MT) * (m.BYP / mi.MT);
     const double simd_hz = (double)arch.n_cu * arch.simd_per_cu * arch.clock_hz;
-    const double t_overhead = (double)nblocks * nkb * W * 700.0 / simd_hz;
-    m.t_mfma = (n_mfma * mi.cycles / simd_hz + t_overhead) / simd_busy;
+    // issue cycles next to the MFMAs, per wavefront and K block: loop, barrier and LDS operand reads
+    // (~250) plus load, address and LDS-store instructions for every slice element the lane stages
+    // (~10 each).  Calibrated on TCCG-22: 96x96x8 tiles on 4 wavefronts measured 72 % of MFMA peak
+    // (6 elements per lane), 48x96x48 tiles on 2 wavefronts 59 % (54 per lane and one wavefront per SIMD).
+    const double t_overhead = (double)nblocks * nkb * W * (250.0 + 10.0 * slots) / simd_hz;
+    // an LDS-fed MFMA loop needs co-resident wavefronts to cover LDS and MFMA latency: measured 68 % of
+    // peak with one wavefront per SIMD, 84 % with two, little more beyond
+    const double mfma_occ = waves_simd >= 3.0 ? 0.92 : waves_simd >= 2.0 ? 0.84 : 0.68;
+    m.t_mfma = (n_mfma * mi.cycles / simd_hz / mfma_occ + t_overhead) / simd_busy;
 
     const double lds_reads = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * W * (m.TX + m.TY) * 64.0 * s;
     m.t_lds = (lds_reads + stage_x + stage_y) / (arch.lds_bytes_per_clk_cu * arch.n_cu * arch.clock_hz);
@@ -531,6 +539,42 @@ bool select_mapping(const Contraction& c, DType t, const ArchGfx950& arch, int r
 
 // spec grammar: x=<id>:<tile>,...;y=...;k=...;w=<WX>x<WY>;t=<TX>x<TY>;mi=<n>;lx=<0|1>;ly=<0|1>
 // index ids may also be given by name.
+
+// The panel-resident streaming kernel for this mapping (spec st=<slices requested ahead>): possible when,
+// at the representative extents, every tile is full and unpadded, there are at least two K blocks, the
+// depth divides their number, and the X tile over the whole contracted range plus two Y slices fit the
+// LDS of a CU.  The K-block count becomes a compile-time constant of the emitted object.
+static bool plan_stream(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& m, std::string& err)
+{
+    auto full = [&](const std::vector<int>& ids, const std::vector<int>& tiles) {
+        for (size_t i = 0; i < ids.size(); i++) if (c.indices[ids[i]].rep_size % tiles[i]) return false;
+        return true;
+    };
+    if (m.BX != m.BXP || m.BY != m.BYP || m.BK != m.BKP || !full(m.x_ids, m.x_tiles) || !full(m.y_ids, m.y_tiles) || !full(m.k_ids, m.k_tiles)) {
+        err = "streaming kernel (st=): tiles must divide the representative extents and need no padding";
+        return false;
+    }
+    long long nkb = 1;
+    for (size_t i = 0; i < m.k_ids.size(); i++) nkb *= c.indices[m.k_ids[i]].rep_size / m.k_tiles[i];
+    if (nkb < 2 || nkb > 64 || nkb % m.st_forced) {
+        err = "streaming kernel (st=): needs 2..64 K blocks and a prefetch depth that divides their number (K blocks here: " + std::to_string(nkb) + ")";
+        return false;
+    }
+    const long long lds_x = (m.layx == 0 ? (long long)m.BKP * m.ldx : (long long)m.BXP * m.ldx);
+    const long long lds_y = (m.layy == 0 ? (long long)m.BKP * m.ldy : (long long)m.BYP * m.ldy);
+    const long long bytes = (long long)esize(t) * (nkb * lds_x + 2 * lds_y);
+    if (bytes > arch.lds_bytes_per_cu) {
+        err = "streaming kernel (st=): the X panel needs " + std::to_string(bytes) + " bytes of LDS";
+        return false;
+    }
+    m.STREAM = (int)nkb;
+    m.SPD = m.st_forced;
+    const int waves = m.WX * m.WY;
+    const int bpc = std::max(1, std::min((int)(arch.lds_bytes_per_cu / bytes), arch.max_waves_per_cu / 2 / waves));
+    m.SMW = std::max(1, std::min(4, (bpc * waves + arch.simd_per_cu - 1) / arch.simd_per_cu));
+    return true;
+}
+
 bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, const std::string& spec, Mapping& m, std::string& err)
 {
     m = Mapping();
@@ -577,6 +621,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "pd") m.pd_forced = std::max(1, std::min(8, atoi(val.c_str())));
         else if (key == "cl") m.clds_forced = atoi(val.c_str()) ? 1 : 0;
         else if (key == "no") m.nto_forced = std::max(0, std::min(3, atoi(val.c_str())));
+        else if (key == "st") m.st_forced = std::max(0, std::min(64, atoi(val.c_str())));
         else if (key == "rx") m.RPX = atoi(val.c_str()) ? 1 : 0;
         else if (key == "ry") m.RPY = atoi(val.c_str()) ? 1 : 0;
         else if (key == "lx") lx = atoi(val.c_str());
@@ -590,6 +635,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
     m.layy = ly >= 0 ? ly : ((!m.k_ids.empty() && m.k_ids[0] == fvi(yop) && m.k_tiles[0] >= 4) ? 1 : 0);
     finish_geometry(c, t, m);
     if (!check_mapping(c, t, arch, m, err)) return false;
+    if (m.st_forced > 0 && !plan_stream(c, t, arch, m, err)) return false;
     cost_model(c, t, arch, m);
     return true;
 }
@@ -610,7 +656,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

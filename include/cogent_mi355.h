@@ -121,14 +121,19 @@ void cogent_fill_uniform_f32(float* dst, long long n, unsigned long long seed);
 
 /* Fixed-signature form of the same entry point.  sizes[] holds n_sizes extents
  * in entry-point order; stream is a hipStream_t (NULL = default stream);
- * variant 0 = tiled MFMA kernel, 1 = plain one-lane-per-element kernel whose
- * summation order is the reference host loop's, 2 = tiled (explicit).
+ * variant 0 = the fastest kernel the object holds for these extents (the
+ * panel-resident streaming kernel when it was emitted and the extents give full
+ * tiles and its K-block count, otherwise the tiled MFMA kernel), 1 = plain
+ * one-lane-per-element kernel whose summation order is the reference host
+ * loop's, 2 = the tiled MFMA kernel with one workgroup per output tile.
  * Status codes: 0 ok, 1 null pointer / bad sizes[], 2 negative extent,
  * 3 tensor or grid too large (2^31 elements), 4 launch failed, 5 bad variant. */
 int cogent_run(const int* sizes, int n_sizes, void* C, const void* A, const void* B,
                void* stream, int variant);
 int cogent_num_indices(void);
 const char* cogent_last_error(void);   /* message of the last failing call on this thread */
+int cogent_last_kernel(void);          /* kernel launched by this thread's last call: 0 none, 1 plain, 2 tiled (one
+                                          workgroup per output tile), 3 panel-resident streaming kernel */
 const char* cogent_expression(void);   /* the expression this object was emitted for      */
 const char* cogent_info(void);         /* JSON: the mapping compiled into this object     */
 

@@ -117,6 +117,35 @@ def test_kernel_options_in_a_spec(tools):
     assert odd["swapped_roles"] == 0
 
 
+def test_streaming_kernel_option(tools, tmp_path):
+    """st=<depth>: the object also gets the panel-resident streaming kernel, compiled for the K-block count of the
+    representative extents; refused when tiles do not divide the extents, need padding, the depth does not divide
+    the K-block count, there is a single K block, or the X panel does not fit the LDS of a CU."""
+    text = open(os.path.join(EXPR_DIR, "cfg2_f64.in")).read()
+    base = "x=d:24,c:4;y=b:24,a:4;k=e:8;w=2x2;t=3x3"
+    assert tools.plan(text, "DOUBLE", mapping_spec=base).info["mapping"]["stream"] == [0, 1]
+    m = tools.plan(text, "DOUBLE", mapping_spec=base + ";st=3").info["mapping"]
+    assert m["stream"] == [9, 3] and "st=3" in m["spec"]
+    assert tools.plan(text, "DOUBLE", mapping_spec=m["spec"]).info["mapping"] == m
+    m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:8,a:8;k=e:24;w=3x4;t=3x1;st=1").info["mapping"]
+    assert m["stream"] == [3, 1]
+    out = os.path.join(str(tmp_path), "st.hip")
+    tools.plan(text, "DOUBLE", mapping_spec=base + ";st=3").emit("st_test", out)
+    src = open(out).read()
+    assert "STREAM = 9, SPD = 3, SMW = 2" in src and "cogent_last_kernel" in src
+    for bad, why in ((base + ";st=2", "divides"),                                             # 9 K blocks
+                     ("x=d:24,c:4;y=b:24,a:4;k=e:36;w=2x2;t=3x3;st=3", "divides"),            # 2 K blocks
+                     ("x=d:16,c:4;y=b:24,a:4;k=e:8;w=2x2;t=2x3;st=3", "divide"),              # 16 does not divide 72
+                     ("x=d:72,c:4;y=b:8,a:4;k=e:8;w=6x2;t=3x1;st=3", "LDS")):                 # a 288 x 72 panel of doubles
+        with pytest.raises(Exception) as err:
+            tools.plan(text, "DOUBLE", mapping_spec=bad)
+        assert why in str(err.value), (bad, str(err.value))
+    text4 = open(os.path.join(EXPR_DIR, "cfg4_f32.in")).read()
+    with pytest.raises(Exception) as err:                                                     # one K block
+        tools.plan(text4, "FLOAT", mapping_spec="x=0:24,2:8,4:1;y=1:24,3:2,5:1;k=6:24;w=4x1;t=3x3;mi=1;st=1")
+    assert "K blocks" in str(err.value)
+
+
 BAD_SPECS = [
     "x=d:24;y=b:24,a:4;k=e:8;w=2x2;t=3x3",                # c unmapped
     "x=d:24,c:4,b:2;y=a:4;k=e:8;w=2x2;t=3x3",             # b on the wrong side
