@@ -42,6 +42,15 @@ def load_cache(path=CACHE):
         return json.load(f)
 
 
+def index_order(text):
+    """Index names of an expression in entry-point order: output indices in output order, then the summed ones."""
+    import re
+    line = [l for l in text.splitlines() if l.strip() and not l.lstrip().startswith("#")][0]
+    out = re.search(r"\[([^\]]*)\]", line).group(1).split(",")
+    summed = re.search(r"sum\(([^)]*)\)", line).group(1).split(",")
+    return [v.strip() for v in out[0::2]] + [v.strip() for v in summed[0::2]]
+
+
 def distinct_candidates(cands, top_k):
     """The first top_k candidates that differ in tiles, wavefront grid or instruction (not only in model cost)."""
     seen, out = set(), []
@@ -54,6 +63,49 @@ def distinct_candidates(cands, top_k):
         out.append(c)
         if len(out) >= top_k:
             break
+    return out
+
+
+def stream_shapes(cand, ext, dtype):
+    """Mapping specs shaped for the streaming kernel, built from a candidate's X/Y/K index lists (composite
+    order) and the extents: X tile = whole leading indices up to 96..144 columns (whole rows of C), Y tile 64
+    or 48 rows, K blocks of 24/16/8, many wavefronts with a one-row accumulator tile."""
+    def grow(names, target):
+        tiles, prod = [], 1
+        for n in names:
+            t = max([v for v in range(1, ext[n] + 1) if ext[n] % v == 0 and prod * v <= target and target % (prod * v) == 0], default=1)
+            tiles.append((n, t))
+            prod *= t
+        return tiles, prod
+    out = []
+    xs, ys, ks = [n for n, _ in cand["x"]], [n for n, _ in cand["y"]], [n for n, _ in cand["k"]]
+    x_opts = [(bx,) + grow(xs, bx) for bx in (144, 128, 96, 64, 48, 32)]
+    y_opts = [(by,) + grow(ys, by) for by in (64, 48, 96, 128, 32)]
+    x_opts = [o for o in x_opts if o[2] == o[0]][:2]
+    y_opts = [o for o in y_opts if o[2] == o[0]][:2]
+    for bx, xt, _ in x_opts:
+        for by, yt, _ in y_opts:
+            for kt0 in (24, 16, 8):
+                if not ks or ext[ks[0]] % kt0:
+                    continue
+                nkb = ext[ks[0]] // kt0
+                for n in ks[1:]:
+                    nkb *= ext[n]
+                if not 2 <= nkb <= 64:
+                    continue
+                tx = 3 if (bx // 16) % 3 == 0 else 2 if (bx // 16) % 2 == 0 else 1
+                wx, wy, ty = bx // 16 // tx, by // 16, 1
+                while wx * wy > 16 and wy % 2 == 0:
+                    wy //= 2
+                    ty *= 2
+                if wx * wy > 16:
+                    continue
+                depth = 3 if nkb % 3 == 0 else 2 if nkb % 2 == 0 else 1
+                side = lambda tl: ",".join("%s:%d" % p for p in tl)
+                kside = ",".join("%s:%d" % (n, kt0 if i == 0 else 1) for i, n in enumerate(ks))
+                out.append("x=%s;y=%s;k=%s;w=%dx%d;t=%dx%d;mi=%d;st=%d" % (side(xt), side(yt), kside, wx, wy, tx, ty,
+                                                                          0 if dtype == "DOUBLE" else 1, depth))
+                break
     return out
 
 
@@ -80,11 +132,26 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
         return ";".join(f for f in sp.split(";") if f.split("=")[0] not in keys)
     for c in cands[:6]:
         n = c["model"]["k_steps"] * max(1, c["split_k"])
+        sp = strip(c["spec"], ("sk", "pd", "mw", "lc", "st"))
+        if n == 1 and len(c["k"]) == 1 and c["k"][0][1] in (16, 24, 32, 48):
+            # the whole contracted range in one K block: cut it into blocks of 8 so that there is a stream
+            fields = sp.split(";")
+            kf = [f for f in fields if f.startswith("k=")][0]
+            n = c["k"][0][1] // 8
+            sp = ";".join(kf.rsplit(":", 1)[0] + ":8" if f is kf else f for f in fields)
         if 2 <= n <= 64:
             depth = 3 if n % 3 == 0 else 2 if n % 2 == 0 else 1
-            specs.append(strip(c["spec"], ("sk", "pd", "mw", "lc", "st")) + ";st=%d" % depth)
+            specs.append(sp + ";st=%d" % depth)
+    if cands:
+        plan_info = json.loads(b.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", os.devnull, "--list", "1"]))[0]
+        names = [n for n, _ in plan_info["x"]] + [n for n, _ in plan_info["y"]] + [n for n, _ in plan_info["k"]]
+        order = index_order(open(src).read())
+        if sorted(order) == sorted(names):
+            ext = dict(zip(order, entry["bench_sizes"]))
+            specs += [sp for sp in stream_shapes(cands[0], ext, entry["dtype"]) if sp not in specs]
     if entry.get("map") and entry["map"] not in specs:
         specs.insert(0, entry["map"])                      # the pinned mapping defends its place
+    specs = list(dict.fromkeys(specs))                     # the derived variants of two candidates can coincide
     out = os.path.join(out_root, name)
     os.makedirs(out, exist_ok=True)
     for f in os.listdir(out):
