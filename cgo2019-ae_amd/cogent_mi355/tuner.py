@@ -68,23 +68,38 @@ def distinct_candidates(cands, top_k):
 
 def stream_shapes(cand, ext, dtype):
     """Mapping specs shaped for the streaming kernel, built from a candidate's X/Y/K index lists (composite
-    order) and the extents: X tile = whole leading indices up to 96..144 columns (whole rows of C), Y tile 64
-    or 48 rows, K blocks of 24/16/8, many wavefronts with a one-row accumulator tile."""
+    order) and the extents: whole leading indices up to a target width per side (whole rows of C on the X side,
+    a whole small matrix on either side), K blocks of 24/16/8, many wavefronts with a one-row accumulator tile;
+    each with the X panel resident and with the Y panel resident.  The generator refuses what does not fit."""
     def grow(names, target):
         tiles, prod = [], 1
         for n in names:
-            t = max([v for v in range(1, ext[n] + 1) if ext[n] % v == 0 and prod * v <= target and target % (prod * v) == 0], default=1)
+            t = max([v for v in range(1, ext[n] + 1) if ext[n] % v == 0 and prod * v <= target], default=1)
             tiles.append((n, t))
             prod *= t
         return tiles, prod
+    def grow_balanced(names, target, first):
+        # a short run of the first index, the rest of the width from the following ones
+        tiles, prod = [], 1
+        for i, n in enumerate(names):
+            cap = min(first, target) if i == 0 else target
+            t = max([v for v in range(1, ext[n] + 1) if ext[n] % v == 0 and prod * v <= cap * (1 if i == 0 else 1) and (i == 0 or prod * v <= target)], default=1)
+            tiles.append((n, t))
+            prod *= t
+        return tiles, prod
+    def options(names, targets, balanced=()):
+        seen, out = set(), []
+        for tl, p in [grow(names, tg) for tg in targets] + [grow_balanced(names, tg, f) for tg, f in balanced]:
+            key = tuple(tl)
+            if p >= 16 and key not in seen:
+                seen.add(key)
+                out.append((tl, p))
+        return out[:3]
     out = []
     xs, ys, ks = [n for n, _ in cand["x"]], [n for n, _ in cand["y"]], [n for n, _ in cand["k"]]
-    x_opts = [(bx,) + grow(xs, bx) for bx in (144, 128, 96, 64, 48, 32)]
-    y_opts = [(by,) + grow(ys, by) for by in (64, 48, 96, 128, 32)]
-    x_opts = [o for o in x_opts if o[2] == o[0]][:2]
-    y_opts = [o for o in y_opts if o[2] == o[0]][:2]
-    for bx, xt, _ in x_opts:
-        for by, yt, _ in y_opts:
+    side = lambda tl: ",".join("%s:%d" % p for p in tl)
+    for xt, bx in options(xs, (144, 96)):
+        for yt, by in options(ys, (64, 80), balanced=((64, 8),)):
             for kt0 in (24, 16, 8):
                 if not ks or ext[ks[0]] % kt0:
                     continue
@@ -93,18 +108,21 @@ def stream_shapes(cand, ext, dtype):
                     nkb *= ext[n]
                 if not 2 <= nkb <= 64:
                     continue
-                tx = 3 if (bx // 16) % 3 == 0 else 2 if (bx // 16) % 2 == 0 else 1
-                wx, wy, ty = bx // 16 // tx, by // 16, 1
+                cx, cy = (bx + 15) // 16, (by + 15) // 16            # MFMA tiles per side, padded
+                tx = 3 if cx % 3 == 0 else 2 if cx % 2 == 0 else 1
+                wx, wy, ty = cx // tx, cy, 1
                 while wx * wy > 16 and wy % 2 == 0:
                     wy //= 2
                     ty *= 2
+                if wx * wy > 16 and wx > 1:
+                    tx, wx = cx, 1
                 if wx * wy > 16:
                     continue
                 depth = 3 if nkb % 3 == 0 else 2 if nkb % 2 == 0 else 1
-                side = lambda tl: ",".join("%s:%d" % p for p in tl)
                 kside = ",".join("%s:%d" % (n, kt0 if i == 0 else 1) for i, n in enumerate(ks))
-                out.append("x=%s;y=%s;k=%s;w=%dx%d;t=%dx%d;mi=%d;st=%d" % (side(xt), side(yt), kside, wx, wy, tx, ty,
-                                                                          0 if dtype == "DOUBLE" else 1, depth))
+                base = "x=%s;y=%s;k=%s;w=%dx%d;t=%dx%d;mi=%d;st=%d" % (side(xt), side(yt), kside, wx, wy, tx, ty,
+                                                                      0 if dtype == "DOUBLE" else 1, depth)
+                out += [base, base + ";sy=1"]
                 break
     return out
 
@@ -130,7 +148,7 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     # refuses the ones whose X panel does not fit the LDS or whose tiles do not divide the extents)
     def strip(sp, keys):
         return ";".join(f for f in sp.split(";") if f.split("=")[0] not in keys)
-    for c in cands[:6]:
+    for c in cands[:4]:
         n = c["model"]["k_steps"] * max(1, c["split_k"])
         sp = strip(c["spec"], ("sk", "pd", "mw", "lc", "st"))
         if n == 1 and len(c["k"]) == 1 and c["k"][0][1] in (16, 24, 32, 48):
@@ -141,7 +159,7 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
             sp = ";".join(kf.rsplit(":", 1)[0] + ":8" if f is kf else f for f in fields)
         if 2 <= n <= 64:
             depth = 3 if n % 3 == 0 else 2 if n % 2 == 0 else 1
-            specs.append(sp + ";st=%d" % depth)
+            specs += [sp + ";st=%d" % depth, sp + ";st=%d;sy=1" % depth]
     if cands:
         plan_info = json.loads(b.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", os.devnull, "--list", "1"]))[0]
         names = [n for n, _ in plan_info["x"]] + [n for n, _ in plan_info["y"]] + [n for n, _ in plan_info["k"]]

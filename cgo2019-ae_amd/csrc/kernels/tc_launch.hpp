@@ -75,18 +75,20 @@ inline void tc_launch_variant(bool one_kb, bool ext_full, bool int_full, bool sw
 }
 
 // The panel-resident streaming kernel, when the object carries one (Cfg::STREAM = its K-block count)
-// and this call has full tiles and exactly that many K blocks.  Returns false when the call has to
-// go to the per-tile kernel instead.  The grid is sized so that all workgroups are resident at once:
-// every X-side tile gets as many runs of consecutive Y-side tiles as fill the CUs about once.
+// and this call's extents are multiples of the tiles and give exactly that many K blocks.  Returns false
+// when the call has to go to the per-tile kernel instead.  The grid is sized so that all workgroups are
+// resident at once: every tile of the resident side gets as many runs of consecutive tiles of the other
+// side as fill the CUs about once.
 template <class Cfg>
-inline bool tc_stream_launch(bool ext_full, bool int_full, int64_t nkb, bool swp, hipStream_t stream,
+inline bool tc_stream_launch(bool ext_div, bool int_div, int64_t nkb, bool swp, hipStream_t stream,
                              typename Cfg::T* c, const typename Cfg::T* x, const typename Cfg::T* y, const TcDims& d)
 {
     if constexpr (Cfg::STREAM > 0) {
         typedef typename Cfg::T T;
-        if (!ext_full || !int_full || nkb != Cfg::STREAM) return false;
-        constexpr size_t lds_bytes = sizeof(T) * ((size_t)Cfg::STREAM * lds_elems<Operand<Cfg, 0>, Cfg::BKP>() + 2 * (size_t)lds_elems<Operand<Cfg, 1>, Cfg::BKP>());
-        static_assert(lds_bytes <= 160 * 1024, "X panel does not fit the LDS");
+        if (!ext_div || !int_div || nkb != Cfg::STREAM) return false;
+        constexpr size_t lds_bytes = sizeof(T) * ((size_t)Cfg::STREAM * lds_elems<Operand<Cfg, Cfg::SRES>, Cfg::BKP>() +
+                                                  2 * (size_t)lds_elems<Operand<Cfg, 1 - Cfg::SRES>, Cfg::BKP>());
+        static_assert(lds_bytes <= 160 * 1024, "the resident panel does not fit the LDS");
         static int n_cu = 0;
         if (n_cu == 0) {
             int dev = 0, v = 0;
@@ -108,18 +110,20 @@ inline bool tc_stream_launch(bool ext_full, bool int_full, int64_t nkb, bool swp
         const int by_lds = (int)((160 * 1024) / lds_bytes), by_regs = (Cfg::SMW * 4 * 64) / Cfg::NT;
         const int64_t slots = (int64_t)n_cu * (by_lds < by_regs ? by_lds : (by_regs < 1 ? 1 : by_regs));
         TcStreamDims s;
-        s.nyt = d.nblocks / d.nxt;
-        int64_t runs = slots / d.nxt;                        // runs per X tile: as many as keep the whole grid resident at once
+        const unsigned nyt = d.nblocks / d.nxt;
+        s.nres = Cfg::SRES == 0 ? d.nxt : nyt;
+        s.nstr = Cfg::SRES == 0 ? nyt : d.nxt;
+        int64_t runs = slots / s.nres;                       // runs per resident tile: as many as keep the whole grid resident at once
         if (runs < 1) runs = 1;
-        if (runs > s.nyt) runs = s.nyt;
-        s.run = (unsigned)((s.nyt + runs - 1) / runs);
-        s.nruns = (s.nyt + s.run - 1) / s.run;
-        const dim3 g(d.nxt * s.nruns), b(Cfg::NT);
+        if (runs > s.nstr) runs = s.nstr;
+        s.run = (unsigned)((s.nstr + runs - 1) / runs);
+        s.nruns = (s.nstr + s.run - 1) / s.run;
+        const dim3 g(s.nres * s.nruns), b(Cfg::NT);
         if (swp) hipLaunchKernelGGL((tc_stream_kernel<Cfg, Cfg::SWAP != 0>), g, b, lds_bytes, stream, c, x, y, d, s);
         else     hipLaunchKernelGGL((tc_stream_kernel<Cfg, false>), g, b, lds_bytes, stream, c, x, y, d, s);
         return true;
     } else {
-        (void)ext_full; (void)int_full; (void)nkb; (void)swp; (void)stream; (void)c; (void)x; (void)y; (void)d;
+        (void)ext_div; (void)int_div; (void)nkb; (void)swp; (void)stream; (void)c; (void)x; (void)y; (void)d;
         return false;
     }
 }
@@ -187,26 +191,28 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
         d.ext[i] = sizes[i]; d.nblk[i] = 1;
         d.sC[i] = (int)sC[i]; d.sX[i] = (int)sX[i]; d.sY[i] = (int)sY[i];
     }
-    bool ext_full = (Cfg::BX == Cfg::BXP) && (Cfg::BY == Cfg::BYP);
-    bool int_full = (Cfg::BK == Cfg::BKP);
+    bool ext_div = true, int_div = true;          // every extent a multiple of its tile
     int64_t grid = 1;
     for (int i = 0; i < Cfg::NX; i++) {
         const int id = Cfg::x_id(i), t = Cfg::x_tile(i);
         d.nblk[id] = (sizes[id] + t - 1) / t; grid *= d.nblk[id];
-        if (sizes[id] % t) ext_full = false;
+        if (sizes[id] % t) ext_div = false;
     }
     const int64_t nxt = grid;
     for (int i = 0; i < Cfg::NY; i++) {
         const int id = Cfg::y_id(i), t = Cfg::y_tile(i);
         d.nblk[id] = (sizes[id] + t - 1) / t; grid *= d.nblk[id];
-        if (sizes[id] % t) ext_full = false;
+        if (sizes[id] % t) ext_div = false;
     }
     int64_t nkb = 1;
     for (int i = 0; i < Cfg::NK; i++) {
         const int id = Cfg::k_id(i), t = Cfg::k_tile(i);
         d.nblk[id] = (sizes[id] + t - 1) / t; nkb *= d.nblk[id];
-        if (sizes[id] % t) int_full = false;
+        if (sizes[id] % t) int_div = false;
     }
+    // the unpredicated variants of the per-tile kernel also need tiles without MFMA padding
+    const bool ext_full = ext_div && (Cfg::BX == Cfg::BXP) && (Cfg::BY == Cfg::BYP);
+    const bool int_full = int_div && (Cfg::BK == Cfg::BKP);
     if (grid > lim || nkb > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
     d.nkb = (int)nkb;
     // split K only when there is a K loop to split; the single-K-block kernels ignore Cfg::SK
@@ -256,7 +262,7 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     const dim3 g((unsigned)grid), b(Cfg::NT);
     // swapped MFMA roles with 128-bit C accesses: fp32 only, fastest extent a multiple of 4, C 16-byte aligned
     const bool swp = Cfg::SWAP && (sizes[Cfg::c_id(0)] % 4 == 0) && (((uintptr_t)C & 15) == 0);
-    if (variant == TC_VARIANT_AUTO && tc_stream_launch<Cfg>(ext_full, int_full, nkb, swp, stream, c, x, y, d)) {
+    if (variant == TC_VARIANT_AUTO && tc_stream_launch<Cfg>(ext_div, int_div, nkb, swp, stream, c, x, y, d)) {
         tc_last_kernel() = TC_KERNEL_STREAM;
     } else {
         tc_launch_variant<Cfg>(nkb == 1, ext_full, int_full, swp, g, b, stream, c, x, y, d);

@@ -6,8 +6,8 @@
 // slices, the write-back.  Here a workgroup is persistent over a RUN of output tiles that share
 // their X-side tile:
 //
-//   * the X panel (the X tile over the whole contracted range, NKB slices) is loaded into LDS once
-//     per workgroup and stays;
+//   * the panel of one side (its tile over the whole contracted range, NKB slices; the X panel below)
+//     is loaded into LDS once per workgroup and stays;
 //   * the Y slices of the tiles of the run pass through a two-stage LDS buffer as ONE stream, PD
 //     slices requested ahead in registers, across tile boundaries: the first slices of the next tile
 //     are in flight while the last K blocks of the current tile are contracted;
@@ -16,6 +16,12 @@
 //     matrix instruction's addend, so that a C read has a whole tile time to arrive and no load burst
 //     stands in front of the slice loads in the in-order return path;
 //   * the finished tile is stored while the next one is already being contracted.
+//
+// Either side can be the resident one (RES = 0: the X panel stays and the run walks Y tiles; RES = 1:
+// the Y panel stays and the run walks X tiles): the side to keep is the one whose tile over the whole
+// contracted range fits the LDS and is re-used by many tiles -- with a small matrix on one side that is
+// the whole matrix.  Tiles padded to the MFMA granularity are allowed: the padding rows of the LDS
+// buffers are cleared once and never written, the padding elements of the C tile are skipped.
 //
 // The K-block count NKB is a compile-time constant (the emitter takes it from the representative
 // extents of the expression): every trip of a tile is a copy of its own, which is what lets the
@@ -27,9 +33,10 @@
 namespace cogent {
 
 struct TcStreamDims {
-    unsigned nyt;      // Y-side tiles of the whole output
-    unsigned run;      // consecutive Y-side tiles handled by one workgroup
-    unsigned nruns;    // workgroups per X-side tile
+    unsigned nres;     // tiles of the whole output along the resident side
+    unsigned nstr;     // ... along the streamed side
+    unsigned run;      // consecutive streamed-side tiles handled by one workgroup
+    unsigned nruns;    // workgroups per resident-side tile
 };
 
 extern __shared__ __attribute__((aligned(16))) unsigned char tc_stream_lds[];
@@ -71,21 +78,26 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
     typedef typename MM::Acc Acc;
     typedef Operand<Cfg, 0> OX;
     typedef Operand<Cfg, 1> OY;
+    constexpr int RES = Cfg::SRES;                 // 0: X panel resident, 1: Y panel resident
+    typedef Operand<Cfg, RES> OR;                  // the resident operand
+    typedef Operand<Cfg, 1 - RES> OS;              // the streamed operand
     constexpr int MT = MM::MT, NREG = MM::NREG, KSTEP = MM::KSTEP;
     constexpr int TX = Cfg::TX, TY = Cfg::TY, NT = Cfg::NT;
     constexpr int NKB = Cfg::STREAM, PD = Cfg::SPD;
     static_assert(NKB >= 2 && PD >= 1 && PD <= NKB && NKB % PD == 0, "prefetch depth must divide the K-block count");
-    static_assert(Cfg::BKP == Cfg::BK && Cfg::BXP == Cfg::BX && Cfg::BYP == Cfg::BY, "streaming kernel: unpadded tiles only");
-    constexpr int SLOTS_X = (Cfg::BK * Cfg::BX + NT - 1) / NT;
-    constexpr int SLOTS_Y = (Cfg::BK * Cfg::BY + NT - 1) / NT;
-    constexpr int LDS_X = lds_elems<OX, Cfg::BKP>();
-    constexpr int LDS_Y = lds_elems<OY, Cfg::BKP>();
+    constexpr bool PADDED = (Cfg::BKP != Cfg::BK) || (Cfg::BXP != Cfg::BX) || (Cfg::BYP != Cfg::BY);
+    constexpr int SLOTS_R = (Cfg::BK * OR::BE + NT - 1) / NT;
+    constexpr int SLOTS_S = (Cfg::BK * OS::BE + NT - 1) / NT;
+    constexpr int LDS_R = lds_elems<OR, Cfg::BKP>();
+    constexpr int LDS_S = lds_elems<OS, Cfg::BKP>();
+    constexpr bool NEG_R = (RES == 1) && (Cfg::SIGN < 0);      // "-=" negates the Y operand while it is staged
+    constexpr bool NEG_S = (RES == 0) && (Cfg::SIGN < 0);
     constexpr bool VEC4 = SWP;
     constexpr bool NT_LD = (Cfg::NTC & 1) != 0, NT_ST = (Cfg::NTC & 2) != 0;
     typedef T T4 __attribute__((ext_vector_type(4)));
 
-    T* const lds_x = (T*)tc_stream_lds;            // NKB slices of the X tile
-    T* const lds_y = lds_x + NKB * LDS_X;          // two stages of one Y slice
+    T* const lds_r = (T*)tc_stream_lds;            // NKB slices of the resident tile
+    T* const lds_s = lds_r + NKB * LDS_R;          // two stages of one slice of the streamed operand
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -93,44 +105,38 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
     const int wx = wave % Cfg::WX;
     const int wy = wave / Cfg::WX;
 
-    // ---- this workgroup's X tile and its run of Y tiles
+    // ---- this workgroup's resident tile and its run of streamed-side tiles
     // Workgroups go to the 8 XCDs round-robin and every XCD has its own L2: give XCD x a contiguous
-    // range of (X tile, run) pairs, X tiles fastest, so that tiles that are neighbours along C's fastest
-    // index -- and share the cache lines their rows end in -- are worked on at the same time on one L2.
+    // range of (resident tile, run) pairs, resident tiles fastest, so that neighbouring tiles are worked
+    // on at the same time on one L2.
     unsigned vb;
     {
         const unsigned n = gridDim.x, xcd = blockIdx.x % 8u, idx = blockIdx.x / 8u;
         const unsigned q = n / 8u, r = n % 8u;
         vb = xcd * q + (xcd < r ? xcd : r) + idx;
     }
-    const unsigned xt = vb % d.nxt, rn = vb / d.nxt;
-    unsigned yt = rn * s.run;
-    const unsigned ntiles = (s.nyt - yt) < s.run ? (s.nyt - yt) : s.run;
-    int64_t baseCx = 0, baseX = 0;
-    {
-        unsigned b = xt;
+    const unsigned rt = vb % s.nres, rn = vb / s.nres;
+    unsigned st = rn * s.run;
+    const unsigned ntiles = (s.nstr - st) < s.run ? (s.nstr - st) : s.run;
+    // origin of a tile along one side: offset inside C and inside that side's operand
+    auto side_origin = [&](auto side_t, unsigned t, int64_t& oc, int64_t& oo) {
+        constexpr int SIDE = decltype(side_t)::value;
+        oc = 0; oo = 0;
 #pragma unroll
-        for (int i = 0; i < Cfg::NX; i++) {
-            const int id = Cfg::x_id(i);
+        for (int i = 0; i < (SIDE == 0 ? Cfg::NX : Cfg::NY); i++) {
+            const int id = SIDE == 0 ? Cfg::x_id(i) : Cfg::y_id(i);
+            const int tile = SIDE == 0 ? Cfg::x_tile(i) : Cfg::y_tile(i);
             const unsigned nb = (unsigned)d.nblk[id];
-            const int o = (int)(b % nb) * Cfg::x_tile(i);
-            b /= nb;
-            baseCx += (int64_t)o * d.sC[id];
-            baseX += (int64_t)o * d.sX[id];
-        }
-    }
-    auto y_origin = [&](unsigned t, int64_t& oc, int64_t& oy) {
-        oc = 0; oy = 0;
-#pragma unroll
-        for (int i = 0; i < Cfg::NY; i++) {
-            const int id = Cfg::y_id(i);
-            const unsigned nb = (unsigned)d.nblk[id];
-            const int o = (int)(t % nb) * Cfg::y_tile(i);
+            const int o = (int)(t % nb) * tile;
             t /= nb;
             oc += (int64_t)o * d.sC[id];
-            oy += (int64_t)o * d.sY[id];
+            oo += (int64_t)o * Operand<Cfg, SIDE>::stride(d, id);
         }
     };
+    const std::integral_constant<int, RES> res_side;
+    const std::integral_constant<int, 1 - RES> str_side;
+    int64_t baseCr, baseR;
+    side_origin(res_side, rt, baseCr, baseR);
 
     // ---- offsets of this lane's accumulator elements from a tile origin: the same for every tile
     int cx[TX][SWP ? NREG : 1];
@@ -143,6 +149,8 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
         asm volatile("" : "+v"(part));
         return (unsigned)(cx[tj][SWP ? r : 0] + part) * (unsigned)sizeof(T);
     };
+    // padded tiles: the accumulator elements that fall into the padding have no place in C
+    auto c_ok = [&](int ti, int tj, int r) -> bool { return !PADDED || (cx[tj][SWP ? r : 0] >= 0 && cy[ti][SWP ? 0 : r] >= 0); };
 
     Acc cpre[TY][TX];       // the C tile that the next first K block starts from
     Acc acc[TY][TX];
@@ -150,13 +158,18 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
         if (VEC4) {
 #pragma unroll
             for (int g = 0; g < NREG / 4; g++) {
-                const T4 v = c_load<NT_LD>((const T4*)((const char*)base + c_off(ti, tj, 4 * g)));
+                T4 v = {(T)0, (T)0, (T)0, (T)0};
+                if (c_ok(ti, tj, 4 * g)) v = c_load<NT_LD>((const T4*)((const char*)base + c_off(ti, tj, 4 * g)));
 #pragma unroll
                 for (int e = 0; e < 4; e++) cpre[ti][tj][4 * g + e] = v[e];
             }
         } else {
 #pragma unroll
-            for (int r = 0; r < NREG; r++) cpre[ti][tj][r] = c_load<NT_LD>((const T*)((const char*)base + c_off(ti, tj, r)));
+            for (int r = 0; r < NREG; r++) {
+                T v = (T)0;
+                if (c_ok(ti, tj, r)) v = c_load<NT_LD>((const T*)((const char*)base + c_off(ti, tj, r)));
+                cpre[ti][tj][r] = v;
+            }
         }
     };
     auto c_write = [&](T* base, int ti, int tj) {
@@ -166,45 +179,52 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
                 T4 v;
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = acc[ti][tj][4 * g + e];
-                c_store<NT_ST>(v, (T4*)((char*)base + c_off(ti, tj, 4 * g)));
+                if (c_ok(ti, tj, 4 * g)) c_store<NT_ST>(v, (T4*)((char*)base + c_off(ti, tj, 4 * g)));
             }
         } else {
 #pragma unroll
-            for (int r = 0; r < NREG; r++) c_store<NT_ST>(acc[ti][tj][r], (T*)((char*)base + c_off(ti, tj, r)));
+            for (int r = 0; r < NREG; r++)
+                if (c_ok(ti, tj, r)) c_store<NT_ST>(acc[ti][tj][r], (T*)((char*)base + c_off(ti, tj, r)));
         }
     };
 
-    // ---- prologue: first C tile, the X panel, the first PD slices of the Y stream
-    int64_t oc, oy;
-    y_origin(yt, oc, oy);
-    T* Cb = C + uniform64(baseCx + oc);
-    const T* Yb = Y + uniform64(oy);
-    const T* Xb = X + uniform64(baseX);
-    KWalk<Cfg, 1> ky;       // the K block of the next slice to request
-    ky.reset();
-    T ry[PD][SLOTS_Y];
+    // ---- prologue: the resident panel, the first PD slices of the stream, the first C tile
+    if (PADDED) {
+        // the staging never writes the padding rows and columns of the LDS buffers: clear everything once
+        for (int i = tid; i < NKB * LDS_R + 2 * LDS_S; i += NT) lds_r[i] = (T)0;
+        __syncthreads();
+    }
+    int64_t oc, oo;
+    side_origin(str_side, st, oc, oo);
+    T* Cb = C + uniform64(baseCr + oc);
+    const T* const Rsrc = (RES == 0 ? X : Y) + uniform64(baseR);
+    const T* const Ssrc = (RES == 0 ? Y : X);
+    const T* Sb = Ssrc + uniform64(oo);
+    KWalk<Cfg, 1 - RES> ks;       // the K block of the next slice to request
+    ks.reset();
+    T rs[PD][SLOTS_S];
     {
-        // The panel in groups of XG slices, all loads of a group in flight together (the accumulators
-        // are not live yet, so the registers are there).  The requests for the first Y slices and for
-        // the first C tile follow the last group's: loads return in order, and the panel and the slices
-        // come from L2 while C comes from HBM.
-        constexpr int XREG = SLOTS_X * (int)sizeof(T) / 4;
-        constexpr int XG = (NKB * XREG <= 96) ? NKB : (96 / XREG < 1 ? 1 : 96 / XREG);
-        constexpr int NG = (NKB + XG - 1) / XG;
-        KWalk<Cfg, 0> kx;
-        kx.reset();
+        // The panel in groups of RG slices, all loads of a group in flight together (the accumulators
+        // are not live yet, so the registers are there).  The requests for the first slices of the stream
+        // and for the first C tile follow the last group's: loads return in order, and the panel and the
+        // slices come from L2 while C comes from HBM.
+        constexpr int RREG = SLOTS_R * (int)sizeof(T) / 4;
+        constexpr int RG = (NKB * RREG <= 96) ? NKB : (96 / RREG < 1 ? 1 : 96 / RREG);
+        constexpr int NG = (NKB + RG - 1) / RG;
+        KWalk<Cfg, RES> kr;
+        kr.reset();
         static_for<NG>([&](auto gt) {
-            constexpr int j0 = decltype(gt)::value * XG;
-            constexpr int n = (NKB - j0) < XG ? (NKB - j0) : XG;
-            T rx[n][SLOTS_X];
+            constexpr int j0 = decltype(gt)::value * RG;
+            constexpr int n = (NKB - j0) < RG ? (NKB - j0) : RG;
+            T rr[n][SLOTS_R];
             static_for<n>([&](auto it) {
-                slice_load<Cfg, OX, true, true>(rx[decltype(it)::value], Xb + uniform64(kx.offset(d)), d, nullptr, tid);
-                kx.next(d);
+                slice_load<Cfg, OR, true, true>(rr[decltype(it)::value], Rsrc + uniform64(kr.offset(d)), d, nullptr, tid);
+                kr.next(d);
             });
             if constexpr (decltype(gt)::value == NG - 1) {
-                static_for<PD>([&](auto st) {
-                    slice_load<Cfg, OY, true, true>(ry[decltype(st)::value], Yb + uniform64(ky.offset(d)), d, nullptr, tid);
-                    ky.next(d);
+                static_for<PD>([&](auto sg) {
+                    slice_load<Cfg, OS, true, true>(rs[decltype(sg)::value], Sb + uniform64(ks.offset(d)), d, nullptr, tid);
+                    ks.next(d);
                 });
 #pragma unroll
                 for (int ti = 0; ti < TY; ti++)
@@ -212,34 +232,34 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
                     for (int tj = 0; tj < TX; tj++) c_read(Cb, ti, tj);
             }
             static_for<n>([&](auto it) {
-                slice_store<Cfg, OX, false>(rx[decltype(it)::value], lds_x + (j0 + decltype(it)::value) * LDS_X, d, tid);
+                slice_store<Cfg, OR, NEG_R>(rr[decltype(it)::value], lds_r + (j0 + decltype(it)::value) * LDS_R, d, tid);
             });
         });
     }
-    slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry[0], lds_y, d, tid);
+    slice_store<Cfg, OS, NEG_S>(rs[0], lds_s, d, tid);
     __syncthreads();
-    int ybuf = 0;           // the LDS stage that holds the current tile's slice 0
+    int sbuf = 0;           // the LDS stage that holds the current tile's slice 0
 
-    // ---- one output tile: NKB trips.  Slice j of the tile is in LDS stage (ybuf + j) % 2 when trip j
+    // ---- one output tile: NKB trips.  Slice j of the tile is in LDS stage (sbuf + j) % 2 when trip j
     // starts; register stage j % PD is free then and takes the request for slice j + PD of the stream.
     auto tile = [&](auto has_next_t) {
         constexpr bool HAS_NEXT = decltype(has_next_t)::value;
         T* Cn = Cb;
-        const T* Yn = Yb;
+        const T* Sn = Sb;
         if (HAS_NEXT) {
-            y_origin(yt + 1, oc, oy);
-            Cn = C + uniform64(baseCx + oc);
-            Yn = Y + uniform64(oy);
+            side_origin(str_side, st + 1, oc, oo);
+            Cn = C + uniform64(baseCr + oc);
+            Sn = Ssrc + uniform64(oo);
         }
         static_for<NKB>([&](auto jt) {
             constexpr int j = decltype(jt)::value;
             constexpr int S = j % PD;
             if constexpr (j + PD < NKB) {
-                slice_load<Cfg, OY, true, true>(ry[S], Yb + uniform64(ky.offset(d)), d, nullptr, tid);
-                ky.next(d);
+                slice_load<Cfg, OS, true, true>(rs[S], Sb + uniform64(ks.offset(d)), d, nullptr, tid);
+                ks.next(d);
             } else if constexpr (HAS_NEXT) {
-                slice_load<Cfg, OY, true, true>(ry[S], Yn + uniform64(ky.offset(d)), d, nullptr, tid);
-                ky.next(d);
+                slice_load<Cfg, OS, true, true>(rs[S], Sn + uniform64(ks.offset(d)), d, nullptr, tid);
+                ks.next(d);
             }
             // the next tile's C, spread over trips 1 .. NKB-1 (trip 0 still reads these registers)
             if constexpr (HAS_NEXT && j >= 1) {
@@ -248,8 +268,10 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
                     if constexpr (1 + (c * (NKB - 1)) / (TY * TX) == j) c_read(Cn, c / TX, c % TX);
                 });
             }
-            const T* lx = lds_x + j * LDS_X;
-            const T* ly = lds_y + (NKB % 2 == 0 ? (j & 1) : (ybuf ^ (j & 1))) * LDS_Y;
+            const T* lr = lds_r + j * LDS_R;
+            const T* ls = lds_s + (NKB % 2 == 0 ? (j & 1) : (sbuf ^ (j & 1))) * LDS_S;
+            const T* lx = RES == 0 ? lr : ls;
+            const T* ly = RES == 0 ? ls : lr;
 #pragma unroll
             for (int k4 = 0; k4 < Cfg::BKP / KSTEP; k4++) {
                 const int kk = k4 * KSTEP + lane / MT;
@@ -267,8 +289,8 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
                     }
             }
             if constexpr (j + 1 < NKB || HAS_NEXT) {
-                T* dst = lds_y + (NKB % 2 == 0 ? ((j + 1) & 1) : (ybuf ^ ((j + 1) & 1))) * LDS_Y;
-                slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry[(j + 1) % PD], dst, d, tid);
+                T* dst = lds_s + (NKB % 2 == 0 ? ((j + 1) & 1) : (sbuf ^ ((j + 1) & 1))) * LDS_S;
+                slice_store<Cfg, OS, NEG_S>(rs[(j + 1) % PD], dst, d, tid);
                 __syncthreads();
             }
         });
@@ -277,8 +299,8 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
 #pragma unroll
             for (int tj = 0; tj < TX; tj++) c_write(Cb, ti, tj);
         if (HAS_NEXT) {
-            Cb = Cn; Yb = Yn; yt++;
-            if (NKB % 2) ybuf ^= 1;
+            Cb = Cn; Sb = Sn; st++;
+            if (NKB % 2) sbuf ^= 1;
         }
     };
 

@@ -71,6 +71,7 @@ std::string Mapping::spec() const
     if (clds_forced >= 0) o << ";cl=" << clds_forced;
     if (nto_forced >= 0) o << ";no=" << nto_forced;
     if (st_forced > 0) o << ";st=" << st_forced;
+    if (SRES) o << ";sy=1";
     if (RPX) o << ";rx=1";
     if (RPY) o << ";ry=1";
     return o.str();
@@ -540,18 +541,19 @@ bool select_mapping(const Contraction& c, DType t, const ArchGfx950& arch, int r
 // spec grammar: x=<id>:<tile>,...;y=...;k=...;w=<WX>x<WY>;t=<TX>x<TY>;mi=<n>;lx=<0|1>;ly=<0|1>
 // index ids may also be given by name.
 
-// The panel-resident streaming kernel for this mapping (spec st=<slices requested ahead>): possible when,
-// at the representative extents, every tile is full and unpadded, there are at least two K blocks, the
-// depth divides their number, and the X tile over the whole contracted range plus two Y slices fit the
-// LDS of a CU.  The K-block count becomes a compile-time constant of the emitted object.
+// The panel-resident streaming kernel for this mapping (spec st=<slices requested ahead>, sy=1 to keep the
+// Y panel instead of the X panel): possible when, at the representative extents, every extent is a multiple
+// of its tile, there are at least two K blocks, the depth divides their number, and the resident tile over
+// the whole contracted range plus two slices of the other operand fit the LDS of a CU.  The K-block count
+// becomes a compile-time constant of the emitted object.
 static bool plan_stream(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& m, std::string& err)
 {
     auto full = [&](const std::vector<int>& ids, const std::vector<int>& tiles) {
         for (size_t i = 0; i < ids.size(); i++) if (c.indices[ids[i]].rep_size % tiles[i]) return false;
         return true;
     };
-    if (m.BX != m.BXP || m.BY != m.BYP || m.BK != m.BKP || !full(m.x_ids, m.x_tiles) || !full(m.y_ids, m.y_tiles) || !full(m.k_ids, m.k_tiles)) {
-        err = "streaming kernel (st=): tiles must divide the representative extents and need no padding";
+    if (!full(m.x_ids, m.x_tiles) || !full(m.y_ids, m.y_tiles) || !full(m.k_ids, m.k_tiles)) {
+        err = "streaming kernel (st=): tiles must divide the representative extents";
         return false;
     }
     long long nkb = 1;
@@ -562,9 +564,9 @@ static bool plan_stream(const Contraction& c, DType t, const ArchGfx950& arch, M
     }
     const long long lds_x = (m.layx == 0 ? (long long)m.BKP * m.ldx : (long long)m.BXP * m.ldx);
     const long long lds_y = (m.layy == 0 ? (long long)m.BKP * m.ldy : (long long)m.BYP * m.ldy);
-    const long long bytes = (long long)esize(t) * (nkb * lds_x + 2 * lds_y);
+    const long long bytes = (long long)esize(t) * (m.SRES ? nkb * lds_y + 2 * lds_x : nkb * lds_x + 2 * lds_y);
     if (bytes > arch.lds_bytes_per_cu) {
-        err = "streaming kernel (st=): the X panel needs " + std::to_string(bytes) + " bytes of LDS";
+        err = "streaming kernel (st=): the resident panel needs " + std::to_string(bytes) + " bytes of LDS";
         return false;
     }
     m.STREAM = (int)nkb;
@@ -622,6 +624,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "cl") m.clds_forced = atoi(val.c_str()) ? 1 : 0;
         else if (key == "no") m.nto_forced = std::max(0, std::min(3, atoi(val.c_str())));
         else if (key == "st") m.st_forced = std::max(0, std::min(64, atoi(val.c_str())));
+        else if (key == "sy") m.SRES = atoi(val.c_str()) ? 1 : 0;
         else if (key == "rx") m.RPX = atoi(val.c_str()) ? 1 : 0;
         else if (key == "ry") m.RPY = atoi(val.c_str()) ? 1 : 0;
         else if (key == "lx") lx = atoi(val.c_str());
@@ -656,7 +659,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"stream_resident\": \"" << (m.SRES ? "y" : "x") << "\", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

@@ -129,6 +129,13 @@ def test_streaming_kernel_option(tools, tmp_path):
     assert tools.plan(text, "DOUBLE", mapping_spec=m["spec"]).info["mapping"] == m
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:8,a:8;k=e:24;w=3x4;t=3x1;st=1").info["mapping"]
     assert m["stream"] == [3, 1]
+    assert m["stream_resident"] == "x"
+    m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:8,a:8;k=e:24;w=3x4;t=3x1;st=3;sy=1").info["mapping"]
+    assert m["stream_resident"] == "y" and "sy=1" in m["spec"]
+    # tiles padded to the MFMA granularity are allowed (a 72-wide side runs as 80)
+    text9 = open(os.path.join(EXPR_DIR, "tccg_09.in")).read()
+    m = tools.plan(text9, "DOUBLE", mapping_spec="x=a:72;y=b:8,c:8,d:1;k=e:24;w=1x4;t=5x1;st=3").info["mapping"]
+    assert m["stream"] == [3, 3] and m["padded"][0] == 80 and m["block_tile"][0] == 72
     out = os.path.join(str(tmp_path), "st.hip")
     tools.plan(text, "DOUBLE", mapping_spec=base + ";st=3").emit("st_test", out)
     src = open(out).read()
