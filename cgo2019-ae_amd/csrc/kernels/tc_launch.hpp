@@ -89,26 +89,30 @@ inline bool tc_stream_launch(bool ext_div, bool int_div, int64_t nkb, bool swp, 
         constexpr size_t lds_bytes = sizeof(T) * ((size_t)Cfg::STREAM * lds_elems<Operand<Cfg, Cfg::SRES>, Cfg::BKP>() +
                                                   2 * (size_t)lds_elems<Operand<Cfg, 1 - Cfg::SRES>, Cfg::BKP>());
         static_assert(lds_bytes <= 160 * 1024, "the resident panel does not fit the LDS");
-        static int n_cu = 0;
-        if (n_cu == 0) {
-            int dev = 0, v = 0;
-            if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 1) {
+        // per device: its CU count, and the kernel's dynamic-LDS limit raised once (neither is a stream
+        // operation, so a call that is being captured into a graph may do them)
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return false; }
+        static int n_cu[64] = {0};
+        static bool configured[64][2] = {{false, false}};
+        if (n_cu[dev] == 0) {
+            int v = 0;
+            if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 1) {
                 (void)hipGetLastError();
                 return false;
             }
-            n_cu = v;
+            n_cu[dev] = v;
         }
-        const void* fn = swp ? (const void*)&tc_stream_kernel<Cfg, Cfg::SWAP != 0> : (const void*)&tc_stream_kernel<Cfg, false>;
-        static bool configured[2] = {false, false};
-        if (!configured[swp ? 1 : 0]) {
+        if (!configured[dev][swp ? 1 : 0]) {
+            const void* fn = swp ? (const void*)&tc_stream_kernel<Cfg, Cfg::SWAP != 0> : (const void*)&tc_stream_kernel<Cfg, false>;
             if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) {
                 (void)hipGetLastError();
                 return false;
             }
-            configured[swp ? 1 : 0] = true;
+            configured[dev][swp ? 1 : 0] = true;
         }
         const int by_lds = (int)((160 * 1024) / lds_bytes), by_regs = (Cfg::SMW * 4 * 64) / Cfg::NT;
-        const int64_t slots = (int64_t)n_cu * (by_lds < by_regs ? by_lds : (by_regs < 1 ? 1 : by_regs));
+        const int64_t slots = (int64_t)n_cu[dev] * (by_lds < by_regs ? by_lds : (by_regs < 1 ? 1 : by_regs));
         TcStreamDims s;
         const unsigned nyt = d.nblocks / d.nxt;
         s.nres = Cfg::SRES == 0 ? d.nxt : nyt;

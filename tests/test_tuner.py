@@ -21,6 +21,41 @@ def test_distinct_candidates_skip_repeats_of_one_tiling():
     assert [c["spec"] for c in tuner.distinct_candidates(cands, 2)] == ["a", "b"]
 
 
+def test_index_order_is_the_entry_points_size_order():
+    from cogent_mi355 import tuner
+    assert tuner.index_order("# note\nt3 [d,72,c,72,b,72,a,72] += sum(e,72) * t2 [b,e,a] * v2 [c,e,d];\n") == ["d", "c", "b", "a", "e"]
+    assert tuner.index_order("t3 [a,48,b,48] -= sum(e,8,f,6) * t2 [a,e,f] * v2 [f,b,e];") == ["a", "b", "e", "f"]
+
+
+def test_stream_shaped_candidates():
+    """Shapes offered for the streaming kernel: whole rows of C on the X side, a whole small matrix on either side,
+    both panels as the resident one; every one of them is either planned or refused with a message."""
+    import cogent_mi355 as pkg
+    from cogent_mi355 import tuner
+    tools = pkg.HostTools()
+    cand = {"x": [["d", 24], ["c", 4]], "y": [["b", 24], ["a", 4]], "k": [["e", 8]]}
+    ext = dict(zip("dcbae", [72] * 5))
+    specs = tuner.stream_shapes(cand, ext, "DOUBLE")
+    assert "x=d:72,c:2;y=b:8,a:8;k=e:24;w=3x4;t=3x1;mi=0;st=3" in specs             # config 2's pinned mapping
+    assert any(sp.endswith(";sy=1") for sp in specs) and len(specs) == len(set(specs)) <= 12
+    text = pkg.expression_text("cfg2_f64")
+    planned = 0
+    for sp in specs:
+        try:
+            m = tools.plan(text, "DOUBLE", mapping_spec=sp).info["mapping"]
+            assert m["stream"][0] == 3 and m["stream_resident"] == ("y" if sp.endswith("sy=1") else "x")
+            planned += 1
+        except pkg.CogentError as err:
+            assert str(err)
+    assert planned >= 4
+    # one side a 72 x 72 matrix: the whole matrix becomes the panel, 72 padded to 80
+    cand = {"x": [["a", 72]], "y": [["b", 8], ["c", 8], ["d", 1]], "k": [["e", 8]]}
+    specs = tuner.stream_shapes(cand, dict(zip("abcde", [72] * 5)), "DOUBLE")
+    assert any(sp.startswith("x=a:72;y=b:8,c:8,d:1;k=e:24;") for sp in specs)
+    # nothing to offer when there is a single K block at every depth tried, or no summed index
+    assert tuner.stream_shapes({"x": [["a", 64]], "y": [["b", 64]], "k": [["c", 4]]}, {"a": 64, "b": 64, "c": 4}, "FLOAT") == []
+
+
 def test_prepared_set_of_the_build_is_complete():
     """build.py compiles the candidates of its TUNING_SETS; the index names one shared object per candidate."""
     import build
