@@ -226,6 +226,17 @@ __device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const i
     }
 }
 
+extern __shared__ __attribute__((aligned(16))) unsigned char tc_dynamic_lds[];
+
+// Bytes of dynamic LDS a variant of the contraction kernel needs (0: its buffers are static).
+template <class Cfg, bool ONE_KB>
+constexpr size_t tc_mfma_dynamic_lds()
+{
+    typedef typename Cfg::T T;
+    constexpr size_t two = 2 * (size_t)(lds_elems<Operand<Cfg, 0>, Cfg::BKP>() + lds_elems<Operand<Cfg, 1>, Cfg::BKP>()) * sizeof(T);
+    return (!ONE_KB && Cfg::DBUF != 0 && two > 65536 && two <= 160 * 1024) ? two : 0;
+}
+
 // The contraction kernel.  EXT_FULL: every external extent is a multiple of its
 // tile and the tile products need no padding; INT_FULL: the same for the
 // contracted indices.  (The reference picks among four kernels by the same two
@@ -274,18 +285,23 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     constexpr bool PADDED = (Cfg::BKP != Cfg::BK) || (Cfg::BXP != Cfg::BX) || (Cfg::BYP != Cfg::BY);
     // two LDS stages when there is a K loop and both fit the static 64 KB: the next slices are
     // written while other wavefronts still read the current ones, one barrier per K block
-    constexpr int NBUF = (!ONE_KB && 2 * (LDS_X + LDS_Y) * (int)sizeof(T) <= 65536) ? 2 : 1;
+    // Cfg::DBUF: the two stages live in dynamic LDS, which can be larger than the 64 KB a static array may have
+    // (large tiles with deep K blocks, one workgroup per CU anyway): the launcher passes the size.
+    constexpr bool BIG = !ONE_KB && Cfg::DBUF != 0 && 2 * (LDS_X + LDS_Y) * (int)sizeof(T) > 65536 &&
+                         2 * (LDS_X + LDS_Y) * (int)sizeof(T) <= 160 * 1024;
+    constexpr int NBUF = (!ONE_KB && (BIG || 2 * (LDS_X + LDS_Y) * (int)sizeof(T) <= 65536)) ? 2 : 1;
 
     // C tile through LDS (CL): the tile is read from and written to global memory in C's own memory
     // order, 16 bytes per lane and whole lines per wavefront whatever the MFMA lane layout is, and
     // changes hands with the accumulators through a dense copy in LDS that shares the operand buffers.
     // Full tiles without split K only; the other variants of the same object use the direct path.
     constexpr int SK0 = ONE_KB ? 1 : Cfg::SK;
-    constexpr bool CL = (Cfg::CLDS != 0) && EXT_FULL && SK0 == 1 && (ONE_KB || Cfg::LATEC == 0);
+    constexpr bool CL = (Cfg::CLDS != 0) && EXT_FULL && SK0 == 1 && (ONE_KB || Cfg::LATEC == 0) && !BIG;
     constexpr int TILE_VOL = Cfg::BX * Cfg::BY;
     constexpr int LDS_OPS = NBUF * (LDS_X + LDS_Y);
     constexpr int LDS_ALL = (CL && TILE_VOL > LDS_OPS) ? TILE_VOL : LDS_OPS;
-    __shared__ __attribute__((aligned(16))) T lds_all[LDS_ALL];
+    __shared__ __attribute__((aligned(16))) T lds_static[BIG ? 4 : LDS_ALL];
+    T* const lds_all = BIG ? (T*)tc_dynamic_lds : lds_static;
     T* const lds_x_all = lds_all;
     T* const lds_y_all = lds_all + NBUF * LDS_X;
 

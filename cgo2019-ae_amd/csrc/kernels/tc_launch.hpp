@@ -53,10 +53,18 @@ template <class Cfg, bool ONE_KB, bool SWP>
 inline void tc_launch_full_partial(bool ext_full, bool int_full, dim3 g, dim3 b, hipStream_t stream,
                                    typename Cfg::T* c, const typename Cfg::T* x, const typename Cfg::T* y, const TcDims& d)
 {
-    if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, ONE_KB, SWP>),   g, b, 0, stream, c, x, y, d);
-    else if (ext_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false, ONE_KB, SWP>),  g, b, 0, stream, c, x, y, d);
-    else if (int_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true, ONE_KB, SWP>),  g, b, 0, stream, c, x, y, d);
-    else                        hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false, ONE_KB, SWP>), g, b, 0, stream, c, x, y, d);
+    constexpr size_t lds = tc_mfma_dynamic_lds<Cfg, ONE_KB>();
+    if (lds > 0) {
+        const void* fn = ext_full && int_full ? (const void*)&tc_mfma_kernel<Cfg, true, true, ONE_KB, SWP>
+                       : ext_full             ? (const void*)&tc_mfma_kernel<Cfg, true, false, ONE_KB, SWP>
+                       : int_full             ? (const void*)&tc_mfma_kernel<Cfg, false, true, ONE_KB, SWP>
+                                              : (const void*)&tc_mfma_kernel<Cfg, false, false, ONE_KB, SWP>;
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return;   // the launch check reports it
+    }
+    if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, ONE_KB, SWP>),   g, b, lds, stream, c, x, y, d);
+    else if (ext_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false, ONE_KB, SWP>),  g, b, lds, stream, c, x, y, d);
+    else if (int_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, true, ONE_KB, SWP>),  g, b, lds, stream, c, x, y, d);
+    else                        hipLaunchKernelGGL((tc_mfma_kernel<Cfg, false, false, ONE_KB, SWP>), g, b, lds, stream, c, x, y, d);
 }
 
 template <class Cfg>

@@ -39,7 +39,6 @@ struct TcStreamDims {
     unsigned nruns;    // workgroups per resident-side tile
 };
 
-extern __shared__ __attribute__((aligned(16))) unsigned char tc_stream_lds[];
 
 
 // Position of a K block in the contracted range (first composite K index fastest) and the element
@@ -96,7 +95,7 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
     constexpr bool NT_LD = (Cfg::NTC & 1) != 0, NT_ST = (Cfg::NTC & 2) != 0;
     typedef T T4 __attribute__((ext_vector_type(4)));
 
-    T* const lds_r = (T*)tc_stream_lds;            // NKB slices of the resident tile
+    T* const lds_r = (T*)tc_dynamic_lds;            // NKB slices of the resident tile
     T* const lds_s = lds_r + NKB * LDS_R;          // two stages of one slice of the streamed operand
 
     const int tid = threadIdx.x;

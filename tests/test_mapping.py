@@ -98,6 +98,13 @@ def test_kernel_options_in_a_spec(tools):
     m = tools.plan(text, "DOUBLE", mapping_spec=base + ";no=2").info["mapping"]
     assert m["nontemporal_inputs"] == 2 and "no=2" in m["spec"]
     assert tools.plan(text, "DOUBLE", mapping_spec=base).info["mapping"]["nontemporal_inputs"] == 0
+    # db=1: two LDS stages in dynamic LDS when together they exceed the 64 KB a static array may have
+    text22 = open(os.path.join(EXPR_DIR, "tccg_22.in")).read()
+    big = "x=0:24,2:8;y=1:72,3:2;k=5:8,4:2;w=4x3;t=3x3"
+    m0 = tools.plan(text22, "DOUBLE", mapping_spec=big).info["mapping"]
+    m1 = tools.plan(text22, "DOUBLE", mapping_spec=big + ";db=1").info["mapping"]
+    assert m0["dynamic_lds_stages"] == 0 and m1["dynamic_lds_stages"] == 1 and "db=1" in m1["spec"]
+    assert 32768 < m1["lds_bytes"] <= 65536                                    # one stage fits a static array, two do not
     # cl=1: the C tile passes through LDS in memory order (opt-in; refused silently when the tile is too large)
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:8,c:8;y=b:24,a:2;k=e:8;w=2x1;t=2x3;cl=1").info["mapping"]
     assert m["c_through_lds"] == 1 and "cl=1" in m["spec"]
