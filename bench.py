@@ -169,8 +169,8 @@ def main():
                          "(the known-size yardstick the FETCH_SIZE / WRITE_SIZE counter readings are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the contraction shards without "
-              "collectives, see DESIGN.md, but no multi-GPU path is built)" % args.gpus, file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (output tiles are independent, so "
+              "the contraction would shard over the slowest output index without collectives, but no multi-GPU path is built)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch

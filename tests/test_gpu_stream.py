@@ -121,3 +121,29 @@ def test_streaming_kernel_inside_a_captured_graph(tools, oracle):
         g.replay()
         torch.cuda.synchronize()
         assert helpers.rel_error(dC.cpu().numpy(), want2) <= 1e-12, "replay %d" % replay
+
+
+@pytest.mark.parametrize("name,sizes,expect", [("var_cfg4_stream_f32", [24, 24, 8, 2, 2, 1, 24], "stream"),
+                                               ("cfg4_16_f32", [16, 16, 16, 2, 2, 1, 16], "tiled")])
+def test_output_not_16_byte_aligned_takes_the_column_layout(name, sizes, expect, tools, oracle):
+    """fp32 objects read and write C with 128-bit accesses when C is 16-byte aligned; a C pointer that is only
+    element-aligned must fall back to the column layout of the same kernel and give the same result."""
+    import torch
+    import cogent_mi355 as pkg
+    ex = pkg.Expression(name)
+    assert ex.info["swapped_roles"] == 1
+    expr = helpers.parse_expression(pkg.expression_text(name))
+    C, A, B = make_inputs(tools, expr, sizes, np.float32)
+    want = oracle.contract(expr, sizes, C.copy(), A, B)
+    dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    for shift in (0, 1):                                       # elements: 0 = aligned, 1 = 4 bytes off
+        buf = torch.full((C.size + 8,), 777.0, dtype=torch.float32, device="cuda")
+        buf[shift:shift + C.size] = torch.from_numpy(C).cuda()
+        print("[gpu] %s sizes=%s C shifted by %d element(s)" % (name, sizes, shift), flush=True)
+        rc = ex.entry(sizes, buf.data_ptr() + 4 * shift, dA.data_ptr(), dB.data_ptr())
+        torch.cuda.synchronize()
+        assert rc == 0, ex.last_error()
+        assert ex.last_kernel() == expect
+        host = buf.cpu().numpy()
+        assert np.all(host[:shift] == 777.0) and np.all(host[shift + C.size:] == 777.0), "write outside C"
+        assert helpers.rel_error(host[shift:shift + C.size], want) <= TOL["f32"]
