@@ -160,6 +160,8 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
         if 2 <= n <= 64:
             depth = 3 if n % 3 == 0 else 2 if n % 2 == 0 else 1
             specs += [sp + ";st=%d" % depth, sp + ";st=%d;sy=1" % depth]
+    # the three best tilings also with 8/16-byte slice loads (pays on some fp64 shapes, costs on fp32 ones)
+    specs += [sp + ";vl=1" for sp in ([s_ for s_ in extra_specs if "vl=" not in s_] + [c["spec"] for c in cands[:3]])[:3]]
     if cands:
         plan_info = json.loads(b.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", os.devnull, "--list", "1"]))[0]
         names = [n for n, _ in plan_info["x"]] + [n for n, _ in plan_info["y"]] + [n for n, _ in plan_info["k"]]

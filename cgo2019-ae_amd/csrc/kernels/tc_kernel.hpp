@@ -78,6 +78,7 @@ template <class Cfg, int SIDE> struct Operand;
 template <class Cfg> struct Operand<Cfg, 0> {
     static constexpr int R = Cfg::XR, LAY = Cfg::LAYX, LD = Cfg::LDX, BE = Cfg::BX, BEP = Cfg::BXP;
     static constexpr bool NTL = (Cfg::NTO & 1) != 0;      // this input is read once: non-temporal loads
+    static constexpr int VW = Cfg::VWX;                   // elements per global load when the slice's fastest run allows (1: scalar)
     __device__ static __forceinline__ constexpr int id(int j)   { return Cfg::xo_id(j); }
     __device__ static __forceinline__ constexpr int tile(int j) { return Cfg::xo_tile(j); }
     __device__ static __forceinline__ constexpr int isk(int j)  { return Cfg::xo_isk(j); }
@@ -87,6 +88,7 @@ template <class Cfg> struct Operand<Cfg, 0> {
 template <class Cfg> struct Operand<Cfg, 1> {
     static constexpr int R = Cfg::YR, LAY = Cfg::LAYY, LD = Cfg::LDY, BE = Cfg::BY, BEP = Cfg::BYP;
     static constexpr bool NTL = (Cfg::NTO & 2) != 0;
+    static constexpr int VW = Cfg::VWY;
     __device__ static __forceinline__ constexpr int id(int j)   { return Cfg::yo_id(j); }
     __device__ static __forceinline__ constexpr int tile(int j) { return Cfg::yo_tile(j); }
     __device__ static __forceinline__ constexpr int isk(int j)  { return Cfg::yo_isk(j); }
@@ -146,34 +148,68 @@ __device__ __forceinline__ void slice_element(unsigned q, const TcDims& d, const
     loff = lds_addr<Op>(k, e);
 }
 
+// Vector width of an operand's slice loads in a kernel variant: Op::VW consecutive elements of the operand's
+// fastest index per lane (one 8- or 16-byte load) when that index's tile is a multiple of it and the tiles of
+// its class are full in this variant (so that a vector never straddles the edge of the tensor); 1 otherwise.
+template <class Op, bool EXT_FULL, bool INT_FULL>
+constexpr int slice_vw() { return (Op::VW > 1 && Op::tile(0) % Op::VW == 0 && (Op::isk(0) ? INT_FULL : EXT_FULL)) ? Op::VW : 1; }
+// Registers per lane that hold its share of a slice
+template <class Cfg, class Op, int V>
+constexpr int slice_slots() { return V * ((Cfg::BK * Op::BE / V + Cfg::NT - 1) / Cfg::NT); }
+
 template <class Cfg, class Op, bool EXT_FULL, bool INT_FULL, int SLOTS>
 __device__ __forceinline__ void slice_load(typename Cfg::T (&reg)[SLOTS], const typename Cfg::T* __restrict__ src,
                                            const TcDims& d, const int* rem, int tid)
 {
     typedef typename Cfg::T T;
+    constexpr int V = slice_vw<Op, EXT_FULL, INT_FULL>();
+    static_assert(SLOTS == slice_slots<Cfg, Op, V>(), "register count of a slice does not match its vector width");
+    // element alignment only: the vector may start at any element of the tensor
+    typedef T TVec __attribute__((ext_vector_type(V), aligned(sizeof(T))));
     constexpr unsigned E = (unsigned)(Cfg::BK * Op::BE);
 #pragma unroll
-    for (int s = 0; s < SLOTS; s++) {
-        const unsigned q = (unsigned)tid + (unsigned)s * Cfg::NT;
+    for (int s = 0; s < SLOTS / V; s++) {
+        const unsigned q = ((unsigned)tid + (unsigned)s * Cfg::NT) * V;
         unsigned goff; int loff; bool valid;
         slice_element<Op, EXT_FULL, INT_FULL>(q, d, rem, goff, loff, valid);
-        T v = (T)0;
-        if ((E % Cfg::NT == 0 || q < E) && valid) v = c_load<Op::NTL>((const T*)((const char*)src + goff * (unsigned)sizeof(T)));
-        reg[s] = v;
+        const bool take = ((E / V) % Cfg::NT == 0 || q < E) && valid;
+        if constexpr (V == 1) {
+            T v = (T)0;
+            if (take) v = c_load<Op::NTL>((const T*)((const char*)src + goff * (unsigned)sizeof(T)));
+            reg[s] = v;
+        } else {
+            TVec v;
+#pragma unroll
+            for (int e = 0; e < V; e++) v[e] = (T)0;
+            if (take) {
+                const TVec* p = (const TVec*)((const char*)src + goff * (unsigned)sizeof(T));
+                v = Op::NTL ? __builtin_nontemporal_load(p) : *p;
+            }
+#pragma unroll
+            for (int e = 0; e < V; e++) reg[s * V + e] = v[e];
+        }
     }
 }
 
-template <class Cfg, class Op, bool NEGATE, int SLOTS>
+// LDS distance between two elements that are neighbours along the operand's fastest index
+template <class Op>
+constexpr int slice_lds_step() { return Op::isk(0) ? (Op::LAY == 0 ? Op::mul(0) * Op::LD : Op::mul(0)) : (Op::LAY == 0 ? Op::mul(0) : Op::mul(0) * Op::LD); }
+
+template <class Cfg, class Op, bool NEGATE, int V = 1, int SLOTS>
 __device__ __forceinline__ void slice_store(const typename Cfg::T (&reg)[SLOTS], typename Cfg::T* lds,
                                             const TcDims& d, int tid)
 {
     constexpr unsigned E = (unsigned)(Cfg::BK * Op::BE);
+    constexpr int STEP = slice_lds_step<Op>();
 #pragma unroll
-    for (int s = 0; s < SLOTS; s++) {
-        const unsigned q = (unsigned)tid + (unsigned)s * Cfg::NT;
+    for (int s = 0; s < SLOTS / V; s++) {
+        const unsigned q = ((unsigned)tid + (unsigned)s * Cfg::NT) * V;
         unsigned goff; int loff; bool valid;
         slice_element<Op, true, true>(q, d, nullptr, goff, loff, valid);
-        if (E % Cfg::NT == 0 || q < E) lds[loff] = NEGATE ? -reg[s] : reg[s];
+        if ((E / V) % Cfg::NT == 0 || q < E) {
+#pragma unroll
+            for (int e = 0; e < V; e++) lds[loff + e * STEP] = NEGATE ? -reg[s * V + e] : reg[s * V + e];
+        }
     }
 }
 
@@ -278,8 +314,9 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     typedef Operand<Cfg, 1> OY;
     constexpr int MT = MM::MT, NREG = MM::NREG, KSTEP = MM::KSTEP;
     constexpr int TX = Cfg::TX, TY = Cfg::TY, NT = Cfg::NT;
-    constexpr int SLOTS_X = (Cfg::BK * Cfg::BX + NT - 1) / NT;
-    constexpr int SLOTS_Y = (Cfg::BK * Cfg::BY + NT - 1) / NT;
+    constexpr int VX = slice_vw<OX, EXT_FULL, INT_FULL>(), VY = slice_vw<OY, EXT_FULL, INT_FULL>();
+    constexpr int SLOTS_X = slice_slots<Cfg, OX, VX>();
+    constexpr int SLOTS_Y = slice_slots<Cfg, OY, VY>();
     constexpr int LDS_X = lds_elems<OX, Cfg::BKP>();
     constexpr int LDS_Y = lds_elems<OY, Cfg::BKP>();
     constexpr bool PADDED = (Cfg::BKP != Cfg::BK) || (Cfg::BXP != Cfg::BX) || (Cfg::BYP != Cfg::BY);
@@ -521,8 +558,8 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         __builtin_amdgcn_s_waitcnt(0x0F70);
     }
     if (NBUF == 2) {
-        slice_store<Cfg, OX, false>(rx[0], lds_x_all, d, tid);
-        slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry[0], lds_y_all, d, tid);
+        slice_store<Cfg, OX, false, VX>(rx[0], lds_x_all, d, tid);
+        slice_store<Cfg, OY, (Cfg::SIGN < 0), VY>(ry[0], lds_y_all, d, tid);
         __syncthreads();
     }
     // One trip: contract K block kb, whose slices are (NBUF == 2) already in LDS or (NBUF == 1) in
@@ -533,8 +570,8 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         T* lds_y = lds_y_all + (NBUF == 2 ? (kb & 1) * LDS_Y : 0);
         if (NBUF == 1) {
             if (!ONE_KB) __syncthreads();      // previous slices fully consumed
-            slice_store<Cfg, OX, false>(rx[S], lds_x, d, tid);
-            slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry[S], lds_y, d, tid);
+            slice_store<Cfg, OX, false, VX>(rx[S], lds_x, d, tid);
+            slice_store<Cfg, OY, (Cfg::SIGN < 0), VY>(ry[S], lds_y, d, tid);
             __syncthreads();
         }
 
@@ -578,8 +615,8 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
             // the slices of K block kb + 1 go to the other LDS buffer (after the last block: the
             // unused repeat of it, harmless)
             if (more) {
-                slice_store<Cfg, OX, false>(rx[SN], lds_x_all + ((kb + 1) & 1) * LDS_X, d, tid);
-                slice_store<Cfg, OY, (Cfg::SIGN < 0)>(ry[SN], lds_y_all + ((kb + 1) & 1) * LDS_Y, d, tid);
+                slice_store<Cfg, OX, false, VX>(rx[SN], lds_x_all + ((kb + 1) & 1) * LDS_X, d, tid);
+                slice_store<Cfg, OY, (Cfg::SIGN < 0), VY>(ry[SN], lds_y_all + ((kb + 1) & 1) * LDS_Y, d, tid);
             }
             __syncthreads();
         }

@@ -85,8 +85,9 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
     constexpr int NKB = Cfg::STREAM, PD = Cfg::SPD;
     static_assert(NKB >= 2 && PD >= 1 && PD <= NKB && NKB % PD == 0, "prefetch depth must divide the K-block count");
     constexpr bool PADDED = (Cfg::BKP != Cfg::BK) || (Cfg::BXP != Cfg::BX) || (Cfg::BYP != Cfg::BY);
-    constexpr int SLOTS_R = (Cfg::BK * OR::BE + NT - 1) / NT;
-    constexpr int SLOTS_S = (Cfg::BK * OS::BE + NT - 1) / NT;
+    constexpr int VR = slice_vw<OR, true, true>(), VS = slice_vw<OS, true, true>();
+    constexpr int SLOTS_R = slice_slots<Cfg, OR, VR>();
+    constexpr int SLOTS_S = slice_slots<Cfg, OS, VS>();
     constexpr int LDS_R = lds_elems<OR, Cfg::BKP>();
     constexpr int LDS_S = lds_elems<OS, Cfg::BKP>();
     constexpr bool NEG_R = (RES == 1) && (Cfg::SIGN < 0);      // "-=" negates the Y operand while it is staged
@@ -231,11 +232,11 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
                     for (int tj = 0; tj < TX; tj++) c_read(Cb, ti, tj);
             }
             static_for<n>([&](auto it) {
-                slice_store<Cfg, OR, NEG_R>(rr[decltype(it)::value], lds_r + (j0 + decltype(it)::value) * LDS_R, d, tid);
+                slice_store<Cfg, OR, NEG_R, VR>(rr[decltype(it)::value], lds_r + (j0 + decltype(it)::value) * LDS_R, d, tid);
             });
         });
     }
-    slice_store<Cfg, OS, NEG_S>(rs[0], lds_s, d, tid);
+    slice_store<Cfg, OS, NEG_S, VS>(rs[0], lds_s, d, tid);
     __syncthreads();
     int sbuf = 0;           // the LDS stage that holds the current tile's slice 0
 
@@ -289,7 +290,7 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
             }
             if constexpr (j + 1 < NKB || HAS_NEXT) {
                 T* dst = lds_s + (NKB % 2 == 0 ? ((j + 1) & 1) : (sbuf ^ ((j + 1) & 1))) * LDS_S;
-                slice_store<Cfg, OS, NEG_S>(rs[(j + 1) % PD], dst, d, tid);
+                slice_store<Cfg, OS, NEG_S, VS>(rs[(j + 1) % PD], dst, d, tid);
                 __syncthreads();
             }
         });

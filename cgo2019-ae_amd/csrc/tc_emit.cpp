@@ -90,6 +90,11 @@ void emit_cfg_members(std::ostringstream& o, const Contraction& c, DType t, cons
             }
         }
         o << "    static constexpr int " << p << "R = " << op.size() << ";\n";
+        // elements per slice load: as many as 16 bytes hold, when the tile of the operand's fastest index is a multiple
+        const int vmax = (t == DType::F64) ? 2 : 4;
+        const int t0 = tiles.empty() ? 1 : tiles[0];
+        const int vw = !m.VL ? 1 : (t0 % vmax == 0 ? vmax : (t0 % 2 == 0 ? 2 : 1));
+        o << "    static constexpr int VW" << p << " = " << vw << ";\n";
         std::string s(1, (char)tolower(p[0]));
         o << table((s + "o_id").c_str(), ids) << table((s + "o_tile").c_str(), tiles)
           << table((s + "o_isk").c_str(), isk) << table((s + "o_mul").c_str(), mul);

@@ -98,6 +98,10 @@ def test_kernel_options_in_a_spec(tools):
     m = tools.plan(text, "DOUBLE", mapping_spec=base + ";no=2").info["mapping"]
     assert m["nontemporal_inputs"] == 2 and "no=2" in m["spec"]
     assert tools.plan(text, "DOUBLE", mapping_spec=base).info["mapping"]["nontemporal_inputs"] == 0
+    # vl=1: slice loads of 8/16 bytes per lane along the operand's fastest index (opt-in)
+    m = tools.plan(text, "DOUBLE", mapping_spec=base + ";vl=1").info["mapping"]
+    assert m["vector_slice_loads"] == 1 and "vl=1" in m["spec"]
+    assert tools.plan(text, "DOUBLE", mapping_spec=base).info["mapping"]["vector_slice_loads"] == 0
     # db=1: two LDS stages in dynamic LDS when together they exceed the 64 KB a static array may have
     text22 = open(os.path.join(EXPR_DIR, "tccg_22.in")).read()
     big = "x=0:24,2:8;y=1:72,3:2;k=5:8,4:2;w=4x3;t=3x3"
