@@ -264,13 +264,15 @@ __device__ __forceinline__ void c_tile_offsets(int lane, int wx, int wy, const i
 
 extern __shared__ __attribute__((aligned(16))) unsigned char tc_dynamic_lds[];
 
-// Bytes of dynamic LDS a variant of the contraction kernel needs (0: its buffers are static).
+// Bytes of dynamic LDS a variant of the contraction kernel needs (0: its buffers are static): with Cfg::DBUF,
+// whenever two stages do not fit a static array -- two stages if they fit the CU's 160 KB, else the one.
 template <class Cfg, bool ONE_KB>
 constexpr size_t tc_mfma_dynamic_lds()
 {
     typedef typename Cfg::T T;
-    constexpr size_t two = 2 * (size_t)(lds_elems<Operand<Cfg, 0>, Cfg::BKP>() + lds_elems<Operand<Cfg, 1>, Cfg::BKP>()) * sizeof(T);
-    return (!ONE_KB && Cfg::DBUF != 0 && two > 65536 && two <= 160 * 1024) ? two : 0;
+    constexpr size_t one = (size_t)(lds_elems<Operand<Cfg, 0>, Cfg::BKP>() + lds_elems<Operand<Cfg, 1>, Cfg::BKP>()) * sizeof(T);
+    if (ONE_KB || Cfg::DBUF == 0 || 2 * one <= 65536) return 0;
+    return 2 * one <= 160 * 1024 ? 2 * one : one;
 }
 
 // The contraction kernel.  EXT_FULL: every external extent is a multiple of its
@@ -324,9 +326,11 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     // written while other wavefronts still read the current ones, one barrier per K block
     // Cfg::DBUF: the two stages live in dynamic LDS, which can be larger than the 64 KB a static array may have
     // (large tiles with deep K blocks, one workgroup per CU anyway): the launcher passes the size.
-    constexpr bool BIG = !ONE_KB && Cfg::DBUF != 0 && 2 * (LDS_X + LDS_Y) * (int)sizeof(T) > 65536 &&
-                         2 * (LDS_X + LDS_Y) * (int)sizeof(T) <= 160 * 1024;
-    constexpr int NBUF = (!ONE_KB && (BIG || 2 * (LDS_X + LDS_Y) * (int)sizeof(T) <= 65536)) ? 2 : 1;
+    // With Cfg::DBUF a single stage of more than 64 KB (a deep K block of a wide tile) is allowed too, up to the
+    // CU's 160 KB; two stages are used whenever both fit.
+    constexpr int ONE_STAGE = (LDS_X + LDS_Y) * (int)sizeof(T);
+    constexpr bool BIG = tc_mfma_dynamic_lds<Cfg, ONE_KB>() > 0;
+    constexpr int NBUF = (!ONE_KB && (BIG ? 2 * ONE_STAGE <= 160 * 1024 : 2 * ONE_STAGE <= 65536)) ? 2 : 1;
 
     // C tile through LDS (CL): the tile is read from and written to global memory in C's own memory
     // order, 16 bytes per lane and whole lines per wavefront whatever the MFMA lane layout is, and

@@ -213,7 +213,10 @@ bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const 
     const int threads = 64 * m.WX * m.WY;
     if (threads < 64 || threads > arch.max_threads_per_block) { err = "threads per block outside 64..1024"; return false; }
     if (m.BXP < m.BX || m.BYP < m.BY) { err = "wavefront tiling does not cover the block tile"; return false; }
-    if (m.lds_bytes > arch.lds_bytes_per_block) { err = "LDS slices exceed 64 KB per block"; return false; }
+    if (m.lds_bytes > (m.DBUF ? arch.lds_bytes_per_cu : arch.lds_bytes_per_block)) {
+        err = m.DBUF ? "LDS slices exceed the 160 KB of a CU" : "LDS slices exceed 64 KB per block";
+        return false;
+    }
     const int acc_regs = m.TX * m.TY * mi.NREG * (esize(t) / 4);
     // 512 registers per lane and SIMD are shared by the block's wavefronts on that SIMD;
     // the accumulators may take half of a wavefront's share
