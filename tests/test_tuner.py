@@ -96,3 +96,23 @@ def test_measure_times_verified_candidates_and_records_the_fastest(tmp_path):
     assert 20.0 < best["mean_us"] < 500.0                                   # 269 MB of traffic: tens of microseconds
     saved = json.load(open(cache))
     assert saved["cfg5_1_f64.in|DOUBLE|16,16,16,16,16,16,16"]["map"] == best["spec"]
+
+
+def test_every_cached_mapping_belongs_to_a_manifest_entry_and_still_plans():
+    """expressions/tuned.json is keyed by file, element type and sizes: no stale keys, and every cached spec (and every
+    spec pinned in manifest.json) is still accepted by the mapping pass for its expression."""
+    import cogent_mi355 as pkg
+    from cogent_mi355 import tuner
+    tools = pkg.HostTools()
+    entries = pkg.manifest()
+    keys = {tuner.cache_key(e): e for e in entries}
+    cache = tuner.load_cache()
+    assert cache, "empty tuning cache"
+    for key, rec in cache.items():
+        assert key in keys, "stale cache key " + key
+        e = keys[key]
+        m = tools.plan(pkg.expression_text(e["name"]), e["dtype"], mapping_spec=rec["map"]).info["mapping"]
+        assert m["threads"] <= 1024 and rec["mean_us"] > 0
+    for e in entries:
+        if e.get("map"):
+            tools.plan(pkg.expression_text(e["name"]), e["dtype"], mapping_spec=e["map"])
