@@ -16,7 +16,8 @@ pytestmark = pytest.mark.gpu
 TOL = {"f64": 1e-12, "f32": 1e-5}
 STREAMING = ["cfg2_f64", "var_cfg2_stream96_f64", "var_cfg4_stream_f32", "var_stream_2k_f64",
              "var_tccg11_stream_y_f64",      # the Y panel resident, its 72 rows padded to 80
-             "var_tccg09_stream_pad_f64"]    # the X panel resident, its 72 columns padded to 80
+             "var_tccg09_stream_pad_f64",    # the X panel resident, its 72 columns padded to 80
+             "var_cfg4_stream_pad_f32"]      # fp32, 128-bit C accesses, a Y tile of 24 rows padded to 32
 
 
 def _check(name, sizes, tools, oracle, variant=None, expect=None):
