@@ -283,7 +283,16 @@ int tc_group_run(const int* sizes, void* C, const void* const* inputs, const int
         if (grid > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
     }
     ga.nblocks = (unsigned)grid;
-    bool too_large = false;
+    bool too_large = false, too_far = false;
+    const int64_t far = ((int64_t)1 << 32) / (int64_t)sizeof(T) - 4;   // 32-bit byte offsets inside a tile and a slice
+    {
+        int64_t span = 0;
+        for (int j = 0; j < G::CR; j++) {
+            const int id = G::c_id(j);
+            span += (int64_t)((sizes[id] < G::c_tile(j) ? sizes[id] : G::c_tile(j)) - 1) * ga.sC[id];
+        }
+        if (span >= far) too_far = true;
+    }
     int t = 0;
     auto fill = [&](auto term) {
         typedef decltype(term) Term;
@@ -295,10 +304,17 @@ int tc_group_run(const int* sizes, void* C, const void* const* inputs, const int
         for (int j = 0; j < Term::XR; j++) { ta.sX[Term::xo_id(j)] = (int)n; n *= sizes[Term::xo_id(j)]; if (n > lim) too_large = true; }
         n = 1;
         for (int j = 0; j < Term::YR; j++) { ta.sY[Term::yo_id(j)] = (int)n; n *= sizes[Term::yo_id(j)]; if (n > lim) too_large = true; }
+        if (!too_large) {
+            int64_t sx = 0, sy = 0;
+            for (int j = 0; j < Term::XR; j++) { const int id = Term::xo_id(j); sx += (int64_t)((sizes[id] < Term::xo_tile(j) ? sizes[id] : Term::xo_tile(j)) - 1) * ta.sX[id]; }
+            for (int j = 0; j < Term::YR; j++) { const int id = Term::yo_id(j); sy += (int64_t)((sizes[id] < Term::yo_tile(j) ? sizes[id] : Term::yo_tile(j)) - 1) * ta.sY[id]; }
+            if (sx >= far || sy >= far) too_far = true;
+        }
         t++;
     };
     (fill(Terms()), ...);
     if (too_large) return tc_fail(TC_ERR_TOO_LARGE, "a tensor has more than 2^31-1 elements");
+    if (too_far) return tc_fail(TC_ERR_TOO_LARGE, "a tile of this mapping spans 4 GB or more of a tensor (byte offsets inside a tile are 32-bit)");
 
     tc_clear_hip_error();
     hipLaunchKernelGGL((tc_group_kernel<G, Terms...>), dim3((unsigned)grid), dim3(G::NT), 0, stream, (T*)C, ga);

@@ -226,6 +226,19 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     const bool ext_full = ext_div && (Cfg::BX == Cfg::BXP) && (Cfg::BY == Cfg::BYP);
     const bool int_full = int_div && (Cfg::BK == Cfg::BKP);
     if (grid > lim || nkb > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
+    {
+        // The kernels address the elements of a tile and of a slice by 32-bit BYTE offsets from a 64-bit origin:
+        // the farthest element of a tile must lie within 4 GB of its first one.
+        auto clip = [&](int id, int tile) { return (int64_t)((sizes[id] < tile ? sizes[id] : tile) - 1); };
+        int64_t spanC = 0, spanX = 0, spanY = 0;
+        for (int i = 0; i < Cfg::NX; i++) spanC += clip(Cfg::x_id(i), Cfg::x_tile(i)) * sC[Cfg::x_id(i)];
+        for (int i = 0; i < Cfg::NY; i++) spanC += clip(Cfg::y_id(i), Cfg::y_tile(i)) * sC[Cfg::y_id(i)];
+        for (int j = 0; j < Cfg::XR; j++) spanX += clip(Cfg::xo_id(j), Cfg::xo_tile(j)) * sX[Cfg::xo_id(j)];
+        for (int j = 0; j < Cfg::YR; j++) spanY += clip(Cfg::yo_id(j), Cfg::yo_tile(j)) * sY[Cfg::yo_id(j)];
+        const int64_t far = ((int64_t)1 << 32) / (int64_t)sizeof(T) - 4;       // a 16-byte access may start at the last element
+        if (spanC >= far || spanX >= far || spanY >= far)
+            return tc_fail(TC_ERR_TOO_LARGE, "a tile of this mapping spans 4 GB or more of a tensor (byte offsets inside a tile are 32-bit)");
+    }
     d.nkb = (int)nkb;
     // split K only when there is a K loop to split; the single-K-block kernels ignore Cfg::SK
     const int sk = (nkb == 1) ? 1 : Cfg::SK;

@@ -32,6 +32,10 @@ def test_status_codes(tools):
     assert ex.run([4, 5, 6], dC.ptr, dA.ptr, dB.ptr, None, 0) == 1          # wrong number of extents
     # 2^31 elements or more in a tensor: refused before anything is launched
     assert ex.entry([2048, 2048, 1024, 2], dC.ptr, dA.ptr, dB.ptr) == 3 and "2^31" in ex.last_error()
+    # fewer than 2^31 elements, but a tile of the mapping would span more than 4 GB of C (32-bit byte offsets inside a tile)
+    import cogent_mi355
+    pinned = cogent_mi355.Expression("var_cfg1_nto_f64")                    # y = a:16,b:4 over C[c,b,a]
+    assert pinned.entry([32, 1200000, 16, 1], dC.ptr, dA.ptr, dB.ptr) == 3 and "4 GB" in pinned.last_error()
     # an empty index range leaves C as it is and succeeds
     for sizes in ([0, 5, 6, 7], [4, 5, 6, 0]):
         assert ex.entry(sizes, dC.ptr, dA.ptr, dB.ptr) == 0
