@@ -127,7 +127,8 @@ void cogent_fill_uniform_f32(float* dst, long long n, unsigned long long seed);
  * one-lane-per-element kernel whose summation order is the reference host
  * loop's, 2 = the tiled MFMA kernel with one workgroup per output tile.
  * Status codes: 0 ok, 1 null pointer / bad sizes[], 2 negative extent,
- * 3 tensor or grid too large (2^31 elements), 4 launch failed, 5 bad variant. */
+ * 3 tensor or grid too large (2^31 elements, or a tile of the mapping spanning 4 GB or more
+ * of a tensor), 4 launch failed, 5 bad variant. */
 int cogent_run(const int* sizes, int n_sizes, void* C, const void* A, const void* B,
                void* stream, int variant);
 int cogent_num_indices(void);
