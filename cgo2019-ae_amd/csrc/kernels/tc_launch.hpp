@@ -59,7 +59,15 @@ inline void tc_launch_full_partial(bool ext_full, bool int_full, dim3 g, dim3 b,
                        : ext_full             ? (const void*)&tc_mfma_kernel<Cfg, true, false, ONE_KB, SWP>
                        : int_full             ? (const void*)&tc_mfma_kernel<Cfg, false, true, ONE_KB, SWP>
                                               : (const void*)&tc_mfma_kernel<Cfg, false, false, ONE_KB, SWP>;
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return;   // the launch check reports it
+        // once per device and variant: raise the kernel's dynamic-LDS limit (not a stream operation)
+        static bool configured[64][4] = {{false}};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;                  // the launch check reports it
+        bool& done = configured[dev][(ext_full ? 2 : 0) + (int_full ? 1 : 0)];
+        if (!done) {
+            if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return;
+            done = true;
+        }
     }
     if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, ONE_KB, SWP>),   g, b, lds, stream, c, x, y, d);
     else if (ext_full)          hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, false, ONE_KB, SWP>),  g, b, lds, stream, c, x, y, d);
