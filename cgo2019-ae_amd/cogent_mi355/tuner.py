@@ -83,7 +83,7 @@ def stream_shapes(cand, ext, dtype):
         tiles, prod = [], 1
         for i, n in enumerate(names):
             cap = min(first, target) if i == 0 else target
-            t = max([v for v in range(1, ext[n] + 1) if ext[n] % v == 0 and prod * v <= cap * (1 if i == 0 else 1) and (i == 0 or prod * v <= target)], default=1)
+            t = max([v for v in range(1, ext[n] + 1) if ext[n] % v == 0 and prod * v <= cap], default=1)
             tiles.append((n, t))
             prod *= t
         return tiles, prod
@@ -163,8 +163,7 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     # the three best tilings also with 8/16-byte slice loads (pays on some fp64 shapes, costs on fp32 ones)
     specs += [sp + ";vl=1" for sp in ([s_ for s_ in extra_specs if "vl=" not in s_] + [c["spec"] for c in cands[:3]])[:3]]
     if cands:
-        plan_info = json.loads(b.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", os.devnull, "--list", "1"]))[0]
-        names = [n for n, _ in plan_info["x"]] + [n for n, _ in plan_info["y"]] + [n for n, _ in plan_info["k"]]
+        names = [n for side in ("x", "y", "k") for n, _ in cands[0][side]]
         order = index_order(open(src).read())
         if sorted(order) == sorted(names):
             ext = dict(zip(order, entry["bench_sizes"]))
