@@ -171,6 +171,8 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     # the streaming kernel reads and writes every element of C once, far apart in time: non-temporal C accesses
     # pay there on many shapes whose rows are not whole lines (where the per-tile kernel loses with them)
     specs += [sp + ";nt=3" for sp in specs if "st=" in sp and "nt=" not in sp]
+    # split K: also with the K shares outermost over the grid, so that the tiles of one share meet in one L2
+    specs += [sp + ";so=1" for sp in specs if "sk=" in sp and "so=" not in sp and "pd=" not in sp]
     if entry.get("map") and entry["map"] not in specs:
         specs.insert(0, entry["map"])                      # the pinned mapping defends its place
     specs = list(dict.fromkeys(specs))                     # the derived variants of two candidates can coincide

@@ -367,8 +367,13 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
             const unsigned q = n / 8u, r = n % 8u;
             b = xcd * q + (xcd < r ? xcd : r) + idx;
         }
-        // split K: SK consecutive workgroups share one output tile, each takes a share of the K blocks
-        if (SK > 1) { ks = b % (unsigned)SK; b /= (unsigned)SK; }
+        // split K: SK consecutive workgroups share one output tile, each takes a share of the K blocks.
+        // SKO: the shares are the outermost level instead, so an XCD's range holds ALL tiles of a few
+        // shares and the operand slices those tiles have in common meet in that XCD's L2.
+        if (SK > 1) {
+            if (Cfg::SKO != 0) { const unsigned nt = d.nblocks / (unsigned)SK; ks = b / nt; b %= nt; }
+            else               { ks = b % (unsigned)SK; b /= (unsigned)SK; }
+        }
         // Within that range walk the tile grid in bands of TILE_GROUP X-tiles (X fastest inside a
         // band, then Y): the ~100 tiles in flight on an XCD then touch a dozen X panels and a dozen
         // Y panels instead of every X panel, and the panels stay in the 4 MB L2 while C streams by.

@@ -63,6 +63,7 @@ std::string Mapping::spec() const
     o << "w=" << WX << "x" << WY << ";t=" << TX << "x" << TY << ";mi=" << MI
       << ";lx=" << layx << ";ly=" << layy;
     if (SK > 1) o << ";sk=" << SK;
+    if (SKO) o << ";so=1";
     if (MINW > 1) o << ";mw=" << MINW;
     if (LATEC) o << ";lc=1";
     if (ntc_forced >= 0) o << ";nt=" << ntc_forced;
@@ -621,6 +622,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
             if (key == "w") { m.WX = a; m.WY = b; } else { m.TX = a; m.TY = b; }
         } else if (key == "mi") m.MI = atoi(val.c_str());
         else if (key == "sk") m.SK = atoi(val.c_str());
+        else if (key == "so") m.SKO = atoi(val.c_str()) ? 1 : 0;
         else if (key == "mw") m.MINW = atoi(val.c_str());
         else if (key == "lc") m.LATEC = atoi(val.c_str()) ? 1 : 0;
         else if (key == "nt") m.ntc_forced = std::max(0, std::min(3, atoi(val.c_str())));
@@ -666,7 +668,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"stream_resident\": \"" << (m.SRES ? "y" : "x") << "\", \"dynamic_lds_stages\": " << m.DBUF << ", \"vector_slice_loads\": " << m.VL << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"split_k_outermost\": " << m.SKO << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"stream_resident\": \"" << (m.SRES ? "y" : "x") << "\", \"dynamic_lds_stages\": " << m.DBUF << ", \"vector_slice_loads\": " << m.VL << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

@@ -108,6 +108,13 @@ def test_kernel_options_in_a_spec(tools):
     m0 = tools.plan(text22, "DOUBLE", mapping_spec=big).info["mapping"]
     m1 = tools.plan(text22, "DOUBLE", mapping_spec=big + ";db=1").info["mapping"]
     assert m0["dynamic_lds_stages"] == 0 and m1["dynamic_lds_stages"] == 1 and "db=1" in m1["spec"]
+    # so=1: with split K, the K shares as the outermost level of the grid (opt-in)
+    text13 = open(os.path.join(EXPR_DIR, "tccg_13.in")).read()
+    sk = "x=a:156;y=b:148;k=d:8,c:2;w=2x2;t=5x5;sk=64"
+    m0 = tools.plan(text13, "DOUBLE", mapping_spec=sk).info["mapping"]
+    m1 = tools.plan(text13, "DOUBLE", mapping_spec=sk + ";so=1").info["mapping"]
+    assert m0["split_k_outermost"] == 0 and m1["split_k_outermost"] == 1 and "so=1" in m1["spec"] and "so=" not in m0["spec"]
+    assert tools.plan(text13, "DOUBLE", mapping_spec=m1["spec"]).info["mapping"] == m1
     assert 32768 < m1["lds_bytes"] <= 65536                                    # one stage fits a static array, two do not
     # cl=1: the C tile passes through LDS in memory order (opt-in; refused silently when the tile is too large)
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:8,c:8;y=b:24,a:2;k=e:8;w=2x1;t=2x3;cl=1").info["mapping"]
