@@ -65,6 +65,7 @@ struct Mapping {
     int WX = 1, WY = 1, TX = 1, TY = 1;       // wavefront grid and MFMA tiles per wavefront
     int MI = 0;                               // 0 f64 16x16x4, 1 f32 16x16x4, 2 f32 32x32x2
     int MINW = 1;                             // resident wavefronts per SIMD asked of the register allocator
+    bool from_spec = false;                   // written by hand or by the tuner (not enumerated): the register check trusts it further
     int SKO = 0;                              // 1 (split K, so=1): the K shares are the grid's outermost level, so the tiles of one share run on one XCD
     int LATEC = 0;                            // 1: load the C tile during the first K block instead of before the loop
     int ntc_forced = -1;                      // -1: decide from the tile shape; 0..3: pinned by a mapping spec (nt=)

@@ -220,10 +220,12 @@ bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const 
     }
     const int acc_regs = m.TX * m.TY * mi.NREG * (esize(t) / 4);
     // 512 registers per lane and SIMD are shared by the block's wavefronts on that SIMD;
-    // the accumulators may take half of a wavefront's share
+    // the accumulators may take half of a wavefront's share.  A mapping given as a spec may take all but
+    // the ~56 registers the rest of the kernel needs at least (whether it then spills is for its author,
+    // or the tuner's clock, to find out).
     const int waves_per_simd = ceil_div(m.WX * m.WY, arch.simd_per_cu);
     const int reg_budget = std::min(512, arch.vgpr_per_lane / waves_per_simd);
-    if (acc_regs > 256 || acc_regs * 2 > reg_budget) { err = "accumulator tiles exceed the register budget per lane"; return false; }
+    if (acc_regs > 256 || (m.from_spec ? acc_regs + 56 > reg_budget : acc_regs * 2 > reg_budget)) { err = "accumulator tiles exceed the register budget per lane"; return false; }
     if (m.layx < 0 || m.layx > 1 || m.layy < 0 || m.layy > 1) { err = "unknown LDS layout"; return false; }
     if (m.SK < 1 || m.SK > 64) { err = "split-K factor outside 1..64"; return false; }
     if (m.MINW < 1 || m.MINW > 8 || m.MINW * ceil_div(m.WX * m.WY, arch.simd_per_cu) > 8) { err = "wavefronts per SIMD outside what a block of this size allows"; return false; }
@@ -647,6 +649,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
     m.layx = lx >= 0 ? lx : ((!m.k_ids.empty() && m.k_ids[0] == fvi(xop) && m.k_tiles[0] >= 4) ? 1 : 0);
     m.layy = ly >= 0 ? ly : ((!m.k_ids.empty() && m.k_ids[0] == fvi(yop) && m.k_tiles[0] >= 4) ? 1 : 0);
     finish_geometry(c, t, m);
+    m.from_spec = true;
     if (!check_mapping(c, t, arch, m, err)) return false;
     if (m.st_forced > 0 && !plan_stream(c, t, arch, m, err)) return false;
     cost_model(c, t, arch, m);
