@@ -144,6 +144,16 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     for sp in deep:
         base = ";".join(f for f in sp.split(";") if not f.startswith("mw="))
         specs += [base + ";pd=2", base + ";pd=2;mw=3"]
+        # ... and with 8-deep K blocks (leading K index 8, the others 1), two in flight: the shallow stages leave
+        # LDS and registers to the accumulators, which won on most MFMA-bound shapes measured
+        fields = [f for f in base.split(";") if f.split("=")[0] not in ("db", "vl")]
+        kf = [f for f in fields if f.startswith("k=")]
+        if kf and kf[0][2:]:
+            ks = [p.split(":")[0] for p in kf[0][2:].split(",")]
+            k8 = "k=" + ",".join("%s:%d" % (n, 8 if i == 0 else 1) for i, n in enumerate(ks))
+            shallow = ";".join(k8 if f is kf[0] else f for f in fields)
+            if shallow != base:
+                specs += [shallow + ";pd=2", shallow + ";pd=2;vl=1"]
     # few K blocks per tile: the best tilings also as the panel-resident streaming kernel (the generator
     # refuses the ones whose X panel does not fit the LDS or whose tiles do not divide the extents)
     def strip(sp, keys):
