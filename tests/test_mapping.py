@@ -181,6 +181,29 @@ BAD_SPECS = [
 ]
 
 
+def test_register_budget_of_specs_and_of_the_enumeration(tools):
+    """The enumeration keeps the accumulators within half a wavefront's register share (at most 16 fp64 MFMA
+    tiles); a spec may take all but 56 registers of the share: 5x5 tiles on four wavefronts (200 of 512) and
+    3x4 on twelve (96 of 170) pass, 3x6 on twelve (144 of 170) and 6x6 on four (288 > 256) do not."""
+    import cogent_mi355
+    text13 = open(os.path.join(EXPR_DIR, "tccg_13.in")).read()
+    plan = tools.plan(text13, "DOUBLE")
+    for c in plan.candidates(300):
+        tx, ty = c["mfma_tiles"] if "mfma_tiles" in c else [int(v) for v in c["spec"].split(";t=")[1].split(";")[0].split("x")]
+        wx, wy = [int(v) for v in c["spec"].split(";w=")[1].split(";")[0].split("x")]
+        share = min(512, 512 // -(-(wx * wy) // 4))
+        assert tx * ty * 8 * 2 <= share, c["spec"]
+    ok = tools.plan(text13, "DOUBLE", mapping_spec="x=a:156;y=b:148;k=d:8,c:2;w=2x2;t=5x5;sk=64").info["mapping"]
+    assert "t=5x5" in ok["spec"]
+    text22 = open(os.path.join(EXPR_DIR, "tccg_22.in")).read()
+    tools.plan(text22, "DOUBLE", mapping_spec="x=a:24,c:8;y=b:24,d:8;k=f:8,e:1;w=4x3;t=3x4;pd=2")
+    for text, bad in ((text22, "x=a:24,c:8;y=b:72,d:4;k=f:8,e:1;w=4x3;t=3x6"),          # 144 of 170
+                      (text13, "x=a:156;y=b:148;k=d:8,c:2;w=2x2;t=6x6;sk=64")):          # 288 accumulator registers
+        with pytest.raises(cogent_mi355.CogentError) as e:
+            tools.plan(text, "DOUBLE", mapping_spec=bad)
+        assert e.value.code == 3 and "register" in str(e.value)
+
+
 @pytest.mark.parametrize("spec", BAD_SPECS)
 def test_impossible_mappings_are_rejected(spec, tools):
     import cogent_mi355
