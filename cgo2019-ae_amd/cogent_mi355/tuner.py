@@ -181,6 +181,13 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     # the streaming kernel reads and writes every element of C once, far apart in time: non-temporal C accesses
     # pay there on many shapes whose rows are not whole lines (where the per-tile kernel loses with them)
     specs += [sp + ";nt=3" for sp in specs if "st=" in sp and "nt=" not in sp]
+    # the C tile staged through LDS in memory order (every C access a whole line), alone and with non-temporal
+    # accesses: pays on HBM-bound shapes whose C rows are not whole lines, most on small tiles
+    for sp in [s_ for s_ in extra_specs if "cl=" not in s_][:2] + [c["spec"] for c in cands[:4]]:
+        if "st=" in sp or "sk=" in sp or "lc=" in sp:
+            continue
+        base = ";".join(f for f in sp.split(";") if f.split("=")[0] not in ("nt", "cl", "db"))
+        specs += [base + ";cl=1", base + ";cl=1;nt=3"]
     # split K: also with the K shares outermost over the grid, so that the tiles of one share meet in one L2
     specs += [sp + ";so=1" for sp in specs if "sk=" in sp and "so=" not in sp and "pd=" not in sp]
     if entry.get("map") and entry["map"] not in specs:
