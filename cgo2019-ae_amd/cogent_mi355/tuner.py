@@ -127,6 +127,31 @@ def stream_shapes(cand, ext, dtype):
     return out
 
 
+def small_tile_shapes(cand, ext, dtype):
+    """Small tiles with the C tile staged through LDS (cl=1), for HBM-bound shapes whose C rows are short: the
+    whole leading X index (when it is at most 32 long) times 4 of the next X index, 16x2 / 8x4 of the first two
+    Y indices, the whole leading K index (at most 32, else 8), four wavefronts.  A 96x32 tile of this kind is
+    what took the 6-D shapes at extents 24/16 from 120-138 us to 106-121 us."""
+    xs, ys, ks = [n for n, _ in cand["x"]], [n for n, _ in cand["y"]], [n for n, _ in cand["k"]]
+    if len(xs) < 2 or len(ys) < 2 or not ks or ext[xs[0]] > 32 or ext[xs[1]] % 4:
+        return []
+    kt = ext[ks[0]] if ext[ks[0]] <= 32 else 8
+    if ext[ks[0]] % kt:
+        return []
+    out = []
+    for y1, y2 in ((16, 2), (8, 4)):
+        if ext[ys[0]] % y1 or ext[ys[1]] % y2:
+            continue
+        nx, ny = -(-(ext[xs[0]] * 4) // 16), -(-(y1 * y2) // 16)
+        if nx % 2 or ny % 2:
+            continue
+        side = lambda names, tiles: ",".join("%s:%d" % (n, tiles[i] if i < len(tiles) else 1) for i, n in enumerate(names))
+        base = "x=%s;y=%s;k=%s;w=2x2;t=%dx%d;mi=%d;cl=1" % (side(xs, [ext[xs[0]], 4]), side(ys, [y1, y2]), side(ks, [kt]),
+                                                          nx // 2, ny // 2, 0 if dtype == "DOUBLE" else 1)
+        out += [base, base + ";nt=3"]
+    return out
+
+
 def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     """Emit and compile the candidates of manifest entry `name`.  Returns the index (list of dicts)."""
     b = _build()
@@ -178,6 +203,7 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
         if sorted(order) == sorted(names):
             ext = dict(zip(order, entry["bench_sizes"]))
             specs += [sp for sp in stream_shapes(cands[0], ext, entry["dtype"]) if sp not in specs]
+            specs += [sp for sp in small_tile_shapes(cands[0], ext, entry["dtype"]) if sp not in specs]
     # the streaming kernel reads and writes every element of C once, far apart in time: non-temporal C accesses
     # pay there on many shapes whose rows are not whole lines (where the per-tile kernel loses with them)
     specs += [sp + ";nt=3" for sp in specs if "st=" in sp and "nt=" not in sp]

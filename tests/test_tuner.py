@@ -116,3 +116,18 @@ def test_every_cached_mapping_belongs_to_a_manifest_entry_and_still_plans():
     for e in entries:
         if e.get("map"):
             tools.plan(pkg.expression_text(e["name"]), e["dtype"], mapping_spec=e["map"])
+
+
+def test_small_tile_shapes():
+    """The 96x32 tile with the C tile through LDS for a 6-D shape at extents 24/16 (TCCG 34: X side a, d, f; Y side
+    b, c, e; contracted g), both Y splits, each with and without non-temporal C; nothing for a long leading index."""
+    from cogent_mi355 import tuner
+    cand = {"x": [["a", 24], ["d", 4], ["f", 1]], "y": [["b", 16], ["c", 8], ["e", 1]], "k": [["g", 8]]}
+    ext = dict(zip("abcdefg", [24, 16, 16, 24, 16, 16, 24]))
+    specs = tuner.small_tile_shapes(cand, ext, "DOUBLE")
+    assert specs == ["x=a:24,d:4,f:1;y=b:16,c:2,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1",
+                     "x=a:24,d:4,f:1;y=b:16,c:2,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1;nt=3",
+                     "x=a:24,d:4,f:1;y=b:8,c:4,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1",
+                     "x=a:24,d:4,f:1;y=b:8,c:4,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1;nt=3"]
+    assert tuner.small_tile_shapes({"x": [["a", 64], ["b", 1]], "y": [["c", 8], ["d", 8]], "k": [["e", 8]]},
+                                   dict(zip("abcde", [72] * 5)), "DOUBLE") == []
