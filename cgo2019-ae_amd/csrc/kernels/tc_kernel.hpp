@@ -436,6 +436,9 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     // the tile in C's memory order: element q of it, as an offset from the tile origin
     constexpr int CV = 16 / (int)sizeof(T);
     typedef T TV __attribute__((ext_vector_type(CV)));
+    // the same vector in global memory: element alignment only, so that C may start at any element of a larger
+    // buffer (the LDS copy is always 16-byte aligned)
+    typedef T TVG __attribute__((ext_vector_type(CV), aligned(sizeof(T))));
     constexpr int NVEC = CL ? (TILE_VOL / CV + NT - 1) / NT : 1;
     auto c_linear = [&](unsigned q) -> unsigned {
         unsigned off = 0;
@@ -453,7 +456,11 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         for (int i = 0; i < NVEC; i++) {
             const unsigned q = (unsigned)(tid + i * NT) * CV;
             if (TILE_VOL % (NT * CV) == 0 || q < (unsigned)TILE_VOL)
-                cv[i] = c_load<(Cfg::NTC & 1) != 0>((const TV*)(Cb + c_linear(q)));
+            {
+                // (not through c_load<>: template deduction would drop the reduced alignment of TVG)
+                const TVG* src = (const TVG*)(Cb + c_linear(q));
+                if ((Cfg::NTC & 1) != 0) cv[i] = __builtin_nontemporal_load(src); else cv[i] = *src;
+            }
         }
 #pragma unroll
         for (int i = 0; i < NVEC; i++) {
@@ -676,7 +683,11 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         for (int i = 0; i < NVEC; i++) {
             const unsigned q = (unsigned)(tid + i * NT) * CV;
             if (TILE_VOL % (NT * CV) == 0 || q < (unsigned)TILE_VOL)
-                c_store<(Cfg::NTC & 2) != 0>(*(const TV*)&lds_all[q], (TV*)(Cb + c_linear(q)));
+            {
+                TVG* dst = (TVG*)(Cb + c_linear(q));
+                const TVG v = *(const TV*)&lds_all[q];
+                if ((Cfg::NTC & 2) != 0) __builtin_nontemporal_store(v, dst); else *dst = v;
+            }
         }
         return;
     }

@@ -11,6 +11,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
+#include <atomic>
 #include "tc_kernel.hpp"
 #include "tc_stream.hpp"
 
@@ -59,14 +60,15 @@ inline void tc_launch_full_partial(bool ext_full, bool int_full, dim3 g, dim3 b,
                        : ext_full             ? (const void*)&tc_mfma_kernel<Cfg, true, false, ONE_KB, SWP>
                        : int_full             ? (const void*)&tc_mfma_kernel<Cfg, false, true, ONE_KB, SWP>
                                               : (const void*)&tc_mfma_kernel<Cfg, false, false, ONE_KB, SWP>;
-        // once per device and variant: raise the kernel's dynamic-LDS limit (not a stream operation)
-        static bool configured[64][4] = {{false}};
+        // once per device and variant: raise the kernel's dynamic-LDS limit (not a stream operation).  Two host
+        // threads may both find the flag clear and both set the same attribute; the flag itself is atomic.
+        static std::atomic<bool> configured[64][4];
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;                  // the launch check reports it
-        bool& done = configured[dev][(ext_full ? 2 : 0) + (int_full ? 1 : 0)];
-        if (!done) {
+        std::atomic<bool>& done = configured[dev][(ext_full ? 2 : 0) + (int_full ? 1 : 0)];
+        if (!done.load(std::memory_order_acquire)) {
             if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return;
-            done = true;
+            done.store(true, std::memory_order_release);
         }
     }
     if (ext_full && int_full)   hipLaunchKernelGGL((tc_mfma_kernel<Cfg, true, true, ONE_KB, SWP>),   g, b, lds, stream, c, x, y, d);
@@ -105,32 +107,35 @@ inline bool tc_stream_launch(bool ext_div, bool int_div, int64_t nkb, bool swp, 
         constexpr size_t lds_bytes = sizeof(T) * ((size_t)Cfg::STREAM * lds_elems<Operand<Cfg, Cfg::SRES>, Cfg::BKP>() +
                                                   2 * (size_t)lds_elems<Operand<Cfg, 1 - Cfg::SRES>, Cfg::BKP>());
         static_assert(lds_bytes <= 160 * 1024, "the resident panel does not fit the LDS");
+        static_assert(Cfg::SK == 1, "the streaming kernel gives every output tile to one workgroup: no split K");
         // per device: its CU count, and the kernel's dynamic-LDS limit raised once (neither is a stream
         // operation, so a call that is being captured into a graph may do them)
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return false; }
-        static int n_cu[64] = {0};
-        static bool configured[64][2] = {{false, false}};
-        if (n_cu[dev] == 0) {
+        static std::atomic<int> n_cu[64];
+        static std::atomic<bool> configured[64][2];
+        if (n_cu[dev].load(std::memory_order_acquire) == 0) {
             int v = 0;
             if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 1) {
                 (void)hipGetLastError();
                 return false;
             }
-            n_cu[dev] = v;
+            n_cu[dev].store(v, std::memory_order_release);
         }
-        if (!configured[dev][swp ? 1 : 0]) {
+        if (!configured[dev][swp ? 1 : 0].load(std::memory_order_acquire)) {
             const void* fn = swp ? (const void*)&tc_stream_kernel<Cfg, Cfg::SWAP != 0> : (const void*)&tc_stream_kernel<Cfg, false>;
             if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) {
                 (void)hipGetLastError();
                 return false;
             }
-            configured[dev][swp ? 1 : 0] = true;
+            configured[dev][swp ? 1 : 0].store(true, std::memory_order_release);
         }
         const int by_lds = (int)((160 * 1024) / lds_bytes), by_regs = (Cfg::SMW * 4 * 64) / Cfg::NT;
-        const int64_t slots = (int64_t)n_cu[dev] * (by_lds < by_regs ? by_lds : (by_regs < 1 ? 1 : by_regs));
+        const int64_t slots = (int64_t)n_cu[dev].load(std::memory_order_relaxed) * (by_lds < by_regs ? by_lds : (by_regs < 1 ? 1 : by_regs));
         TcStreamDims s;
-        const unsigned nyt = d.nblocks / d.nxt;
+        // tiles along the Y side from the tile counts themselves (d.nblocks may carry other grid factors)
+        unsigned nyt = 1;
+        for (int i = 0; i < Cfg::NY; i++) nyt *= (unsigned)d.nblk[Cfg::y_id(i)];
         s.nres = Cfg::SRES == 0 ? d.nxt : nyt;
         s.nstr = Cfg::SRES == 0 ? nyt : d.nxt;
         int64_t runs = slots / s.nres;                       // runs per resident tile: as many as keep the whole grid resident at once

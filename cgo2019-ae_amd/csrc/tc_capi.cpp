@@ -95,7 +95,7 @@ int cogent_plan_emit(const cogent_plan* plan, const char* unique_name, const cha
     return f.good() ? 0 : fail(5, std::string("cannot write '") + out_path + "'");
 }
 
-static std::string g_group_json;
+static thread_local std::string g_group_json;   // per thread, like the error message: concurrent callers do not share it
 
 int cogent_group_emit(const char* text, const char* dtype, const char* tile_spec, const char* unique_name, const char* out_path)
 {

@@ -651,6 +651,8 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
     finish_geometry(c, t, m);
     m.from_spec = true;
     if (!check_mapping(c, t, arch, m, err)) return false;
+    // the streaming kernel gives every output tile to exactly one workgroup: K shares cannot be combined with it
+    if (m.st_forced > 0 && m.SK > 1) { err = "mapping spec: st= (streaming kernel) and sk= (split K) exclude each other"; return false; }
     if (m.st_forced > 0 && !plan_stream(c, t, arch, m, err)) return false;
     cost_model(c, t, arch, m);
     return true;

@@ -124,6 +124,65 @@ def test_streaming_kernel_inside_a_captured_graph(tools, oracle):
         assert helpers.rel_error(dC.cpu().numpy(), want2) <= 1e-12, "replay %d" % replay
 
 
+def test_first_call_of_a_streaming_object_inside_a_capture(tools, oracle, tmp_path):
+    """The first call on a device sizes the kernel's dynamic LDS and reads the CU count; neither is a stream
+    operation, so even a FIRST call may be captured.  A private copy of the object is loaded so that no earlier
+    test of this process has made that first call."""
+    import shutil
+    import torch
+    import cogent_mi355
+    name, sizes = "cfg2_f64", [72, 8, 16, 16, 72]
+    fresh = str(tmp_path / "cfg2_first_call.so")
+    shutil.copy(cogent_mi355.Expression(name).path, fresh)
+    ex = cogent_mi355.Expression(path=fresh)
+    expr = helpers.parse_expression(cogent_mi355.expression_text(name))
+    C, A, B = make_inputs(tools, expr, sizes, np.float64)
+    want = oracle.contract(expr, sizes, C.copy(), A, B)
+    dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), torch.from_numpy(C).cuda()
+    dC0 = dC.clone()
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    print("[gpu] first call of a fresh copy of %s inside a capture, sizes=%s" % (name, sizes), flush=True)
+    with torch.cuda.graph(g, stream=s):
+        st = torch.cuda.current_stream().cuda_stream
+        assert ex.run(sizes, dC.data_ptr(), dA.data_ptr(), dB.data_ptr(), st, 0) == 0, ex.last_error()
+    assert ex.last_kernel() == "stream"
+    for replay in range(3):
+        dC.copy_(dC0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert helpers.rel_error(dC.cpu().numpy(), want) <= 1e-12, "replay %d" % replay
+
+
+@pytest.mark.parametrize("name", ["var_cfg2_clds_f64", "var_cfg4_clds_f32"])
+def test_c_through_lds_with_an_output_that_is_only_element_aligned(name, tools, oracle):
+    """cl=1 objects move full C tiles as 16-byte vectors; C may still start at any ELEMENT of a larger buffer."""
+    import torch
+    import cogent_mi355 as pkg
+    ex = pkg.Expression(name)
+    assert ex.info["c_through_lds"] == 1
+    expr = helpers.parse_expression(pkg.expression_text(name))
+    tiles = _tiles(ex)
+    rep = dict(zip(expr["all_idx"], pkg.manifest_entry(name)["bench_sizes"]))
+    sizes = [min(rep[n], tiles[n] * (2 if j == 0 else 1)) for j, n in enumerate(expr["all_idx"])]       # full tiles: the LDS path
+    np_dtype = np.float64 if ex.dtype == "f64" else np.float32
+    C, A, B = make_inputs(tools, expr, sizes, np_dtype)
+    want = oracle.contract(expr, sizes, C.copy(), A, B)
+    dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    for shift in (0, 1):
+        buf = torch.full((C.size + 8,), 777.0, dtype=torch.float64 if ex.dtype == "f64" else torch.float32, device="cuda")
+        buf[shift:shift + C.size] = torch.from_numpy(C).cuda()
+        print("[gpu] %s sizes=%s C shifted by %d element(s)" % (name, sizes, shift), flush=True)
+        rc = ex.run(sizes, buf.data_ptr() + buf.element_size() * shift, dA.data_ptr(), dB.data_ptr(), None, 2)
+        torch.cuda.synchronize()
+        assert rc == 0, ex.last_error()
+        host = buf.cpu().numpy()
+        assert np.all(host[:shift] == 777.0) and np.all(host[shift + C.size:] == 777.0), "write outside C"
+        assert helpers.rel_error(host[shift:shift + C.size], want) <= TOL[ex.dtype]
+
+
 @pytest.mark.parametrize("name,sizes,expect", [("var_cfg4_stream_f32", [24, 24, 8, 2, 2, 1, 24], "stream"),
                                                ("cfg4_16_f32", [16, 16, 16, 2, 2, 1, 16], "tiled")])
 def test_output_not_16_byte_aligned_takes_the_column_layout(name, sizes, expect, tools, oracle):

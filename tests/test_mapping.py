@@ -161,7 +161,9 @@ def test_streaming_kernel_option(tools, tmp_path):
     for bad, why in ((base + ";st=2", "divides"),                                             # 9 K blocks
                      ("x=d:24,c:4;y=b:24,a:4;k=e:36;w=2x2;t=3x3;st=3", "divides"),            # 2 K blocks
                      ("x=d:16,c:4;y=b:24,a:4;k=e:8;w=2x2;t=2x3;st=3", "divide"),              # 16 does not divide 72
-                     ("x=d:72,c:4;y=b:8,a:4;k=e:8;w=6x2;t=3x1;st=3", "LDS")):                 # a 288 x 72 panel of doubles
+                     ("x=d:72,c:4;y=b:8,a:4;k=e:8;w=6x2;t=3x1;st=3", "LDS"),                  # a 288 x 72 panel of doubles
+                     (base + ";st=3;sk=2", "exclude"),                                         # K shares: every tile has ONE workgroup here
+                     (base + ";sk=3;st=3", "exclude")):
         with pytest.raises(Exception) as err:
             tools.plan(text, "DOUBLE", mapping_spec=bad)
         assert why in str(err.value), (bad, str(err.value))
