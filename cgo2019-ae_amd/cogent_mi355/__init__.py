@@ -170,6 +170,8 @@ class Expression:
         self.lib.cogent_run.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
         self.lib.cogent_run.restype = ctypes.c_int
+        self.lib.cogent_run_noalloc.argtypes = self.lib.cogent_run.argtypes
+        self.lib.cogent_run_noalloc.restype = ctypes.c_int
         for fn in (self.lib.sd_t_d2_fusion_, self.lib.sd_t_d2_fusion_host_):
             fn.argtypes = [ctypes.c_int] * self.n + [ctypes.c_void_p] * 3 + [ctypes.c_int, ctypes.c_int]
             fn.restype = ctypes.c_int
@@ -199,6 +201,11 @@ class Expression:
     def run(self, sizes, c_ptr, a_ptr, b_ptr, stream=None, variant=0):
         arr = (ctypes.c_int * len(sizes))(*[int(s) for s in sizes])
         return self.lib.cogent_run(arr, len(sizes), c_ptr, a_ptr, b_ptr, stream, variant)
+
+    def run_noalloc(self, sizes, c_ptr, a_ptr, b_ptr, stream=None, variant=0):
+        """cogent_run_noalloc: the same call, guaranteed not to allocate (repacked inputs go to the object's static scratch)."""
+        arr = (ctypes.c_int * len(sizes))(*[int(s) for s in sizes])
+        return self.lib.cogent_run_noalloc(arr, len(sizes), c_ptr, a_ptr, b_ptr, stream, variant)
 
 
 class Group:

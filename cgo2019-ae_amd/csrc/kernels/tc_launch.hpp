@@ -156,8 +156,13 @@ inline bool tc_stream_launch(bool ext_div, bool int_div, int64_t nkb, bool swp, 
 // sizes[] holds one extent per index id: output indices in output order, then
 // the contracted indices in sum() order -- the order of the entry point's
 // `int size_*` parameters (cogent/src/codes/kernels/tc_interface.py:1459-1492).
+//
+// no_alloc: the call must not allocate.  A mapping with repacked inputs then puts the copies into the caller's
+// workspace `ext_ws` of `ext_ws_bytes` bytes (the emitted object's static device array) instead of a
+// stream-ordered allocation, and refuses inputs that do not fit it.
 template <class Cfg>
-int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t stream, int variant)
+int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t stream, int variant,
+           void* ext_ws = nullptr, size_t ext_ws_bytes = 0, bool no_alloc = false)
 {
     typedef typename Cfg::T T;
     tc_error_buffer()[0] = 0;
@@ -272,7 +277,14 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
         const int64_t nx = Cfg::X_IS_A ? nA : nB, ny = Cfg::X_IS_A ? nB : nA;
         const int64_t off_y = Cfg::RPX ? ((nx + 31) / 32) * 32 : 0;              // keep the second copy 256-byte aligned
         const int64_t total = off_y + (Cfg::RPY ? ny : 0);
-        if (hipMallocAsync((void**)&ws, (size_t)total * sizeof(T), stream) != hipSuccess || !ws) {
+        if (no_alloc) {
+            if (!ext_ws || (size_t)total * sizeof(T) > ext_ws_bytes) {
+                snprintf(tc_error_buffer(), 256, "the repacked inputs need %lld bytes of scratch, the allocation-free entry point has %lld",
+                         (long long)total * (long long)sizeof(T), (long long)ext_ws_bytes);
+                return TC_ERR_TOO_LARGE;
+            }
+            ws = (T*)ext_ws;
+        } else if (hipMallocAsync((void**)&ws, (size_t)total * sizeof(T), stream) != hipSuccess || !ws) {
             (void)hipGetLastError();
             return tc_fail(TC_ERR_ALLOC, "stream-ordered allocation of the repack buffer failed");
         }
@@ -294,7 +306,7 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
             hipLaunchKernelGGL(tc_repack_kernel<T>, dim3((unsigned)((ny + 255) / 256)), dim3(256), 0, stream, y, ws + off_y, r);
             y = ws + off_y;
         }
-        if (tc_check_launch("repack kernel launch failed") != TC_OK) { (void)hipFreeAsync(ws, stream); return TC_ERR_LAUNCH; }
+        if (tc_check_launch("repack kernel launch failed") != TC_OK) { if (!no_alloc) (void)hipFreeAsync(ws, stream); return TC_ERR_LAUNCH; }
     }
 
     const dim3 g((unsigned)grid), b(Cfg::NT);
@@ -307,7 +319,7 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
         tc_last_kernel() = TC_KERNEL_TILED;
     }
     const int rc = tc_check_launch("tiled kernel launch failed");
-    if (ws && hipFreeAsync(ws, stream) != hipSuccess) { (void)hipGetLastError(); if (rc == TC_OK) return tc_fail(TC_ERR_ALLOC, "stream-ordered free of the repack buffer failed"); }
+    if (ws && !no_alloc && hipFreeAsync(ws, stream) != hipSuccess) { (void)hipGetLastError(); if (rc == TC_OK) return tc_fail(TC_ERR_ALLOC, "stream-ordered free of the repack buffer failed"); }
     return rc;
 }
 

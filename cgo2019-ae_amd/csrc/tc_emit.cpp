@@ -124,6 +124,25 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
     emit_cfg_members(o, c, t, m);
     o << "};\n";
     o << "}  // namespace\n\n";
+    const bool uses_scratch = m.RPX || m.RPY;
+    if (uses_scratch) {
+        o << "// Scratch of the allocation-free entry point (cogent_run_noalloc): the repacked copies of the inputs.\n";
+        o << "// Every GPU this object runs on holds its own copy of the array until the process ends.\n";
+        o << "#define COGENT_SCRATCH_BYTES (16u << 20)\n";
+        o << "static __device__ __align__(256) unsigned char scratch[COGENT_SCRATCH_BYTES];\n\n";
+        o << "// In host code the array's name is only a stand-in, not a device address: the address is asked of the\n";
+        o << "// runtime once per device, with that device current, and kept.\n";
+        o << "static int scratch_address(void** out)\n{\n";
+        o << "    static std::atomic<void*> addr[64];\n";
+        o << "    int dev = 0;\n";
+        o << "    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return cogent::tc_fail(cogent::TC_ERR_LAUNCH, \"no current device\"); }\n";
+        o << "    void* p = addr[dev].load(std::memory_order_acquire);\n";
+        o << "    if (!p) {\n";
+        o << "        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) { (void)hipGetLastError(); return cogent::tc_fail(cogent::TC_ERR_LAUNCH, \"hipGetSymbolAddress(scratch) failed\"); }\n";
+        o << "        addr[dev].store(p, std::memory_order_release);\n";
+        o << "    }\n";
+        o << "    *out = p;\n    return 0;\n}\n\n";
+    }
 
     // parameter lists
     std::ostringstream params, sizes;
@@ -151,6 +170,24 @@ std::string emit_hip_source(const Contraction& c, DType t, const Mapping& m, con
     o << "int cogent_run(const int* sizes, int n_sizes, void* C, const void* A, const void* B, void* stream, int variant)\n{\n";
     o << "    if (!sizes || n_sizes != Cfg::NIDX) return cogent::tc_fail(cogent::TC_ERR_NULL_POINTER, \"sizes[] must hold one extent per index\");\n";
     o << "    return cogent::tc_run<Cfg>(sizes, C, A, B, (hipStream_t)stream, variant);\n}\n\n";
+    o << "// The same call for callers that cannot allocate (code under graph capture, serving loops): no hipMalloc,\n";
+    o << "// hipFree or allocating library routine on any path.  ";
+    if (uses_scratch) {
+        o << "This mapping repacks inputs: the copies go into the\n";
+        o << "// static device array `scratch` (COGENT_SCRATCH_BYTES); inputs that do not fit it are refused with status 3.\n";
+        o << "// Calls that overlap on one GPU share the array and race: one call at a time per device.\n";
+    } else {
+        o << "This mapping needs no scratch memory, so the call\n// is cogent_run itself.\n";
+    }
+    o << "int cogent_run_noalloc(const int* sizes, int n_sizes, void* C, const void* A, const void* B, void* stream, int variant)\n{\n";
+    o << "    if (!sizes || n_sizes != Cfg::NIDX) return cogent::tc_fail(cogent::TC_ERR_NULL_POINTER, \"sizes[] must hold one extent per index\");\n";
+    if (uses_scratch) {
+        o << "    void* ws = nullptr;\n";
+        o << "    if (const int rc = scratch_address(&ws)) return rc;\n";
+        o << "    return cogent::tc_run<Cfg>(sizes, C, A, B, (hipStream_t)stream, variant, ws, (size_t)COGENT_SCRATCH_BYTES, true);\n}\n\n";
+    } else {
+        o << "    return cogent::tc_run<Cfg>(sizes, C, A, B, (hipStream_t)stream, variant, nullptr, 0, true);\n}\n\n";
+    }
     o << "int cogent_" << unique_name << "_run(const int* sizes, int n_sizes, void* C, const void* A, const void* B, void* stream, int variant)\n{\n";
     o << "    return cogent_run(sizes, n_sizes, C, A, B, stream, variant);\n}\n\n";
     o << "int cogent_num_indices(void) { return Cfg::NIDX; }\n";

@@ -131,6 +131,19 @@ void cogent_fill_uniform_f32(float* dst, long long n, unsigned long long seed);
  * of a tensor), 4 launch failed, 5 bad variant. */
 int cogent_run(const int* sizes, int n_sizes, void* C, const void* A, const void* B,
                void* stream, int variant);
+/* cogent_run for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose host caller
+ * allocates and frees on every call, cogent/src/codes/kernels/tc_interface.py:10-101).  Same arguments,
+ * same kernels, same results as cogent_run; no hipMalloc, hipMallocAsync, hipFree or allocating library
+ * routine is called on any path.  The one kernel path with a scratch buffer is a mapping that repacks its
+ * inputs (rx=1 / ry=1): cogent_run takes the copies' memory from the stream-ordered allocator, this entry
+ * point keeps them in a static device array of the object (16 MiB per GPU, held until the process ends)
+ * and returns status 3 with a message naming both sizes when the repacked inputs need more.  Calls that
+ * overlap on one GPU share that array and race: one call at a time per device.  The array's address is
+ * looked up on the first call on each device, which therefore should not itself be captured.  An object
+ * whose mapping needs no scratch memory exports the same symbol; there it is cogent_run. */
+int cogent_run_noalloc(const int* sizes, int n_sizes, void* C, const void* A, const void* B,
+                       void* stream, int variant);
 int cogent_num_indices(void);
 const char* cogent_last_error(void);   /* message of the last failing call on this thread */
 int cogent_last_kernel(void);          /* kernel launched by this thread's last call: 0 none, 1 plain, 2 tiled (one

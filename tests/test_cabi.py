@@ -26,7 +26,7 @@ def test_header_declarations_are_exported():
     for n in host_names:
         assert hasattr(host, n), n
     per_expression = [n for n in names if n not in host_names]
-    assert set(per_expression) == {"cogent_run", "cogent_num_indices", "cogent_last_error", "cogent_last_kernel", "cogent_expression", "cogent_info"}
+    assert set(per_expression) == {"cogent_run", "cogent_run_noalloc", "cogent_num_indices", "cogent_last_error", "cogent_last_kernel", "cogent_expression", "cogent_info"}
 
 
 def test_every_expression_object_exports_the_entry_points():
@@ -36,7 +36,7 @@ def test_every_expression_object_exports_the_entry_points():
         assert os.path.exists(path), "%s not built" % path
         out = subprocess.run(["nm", "-D", "--defined-only", path], stdout=subprocess.PIPE, text=True, check=True).stdout
         syms = {l.split()[-1] for l in out.splitlines() if l.strip()}
-        for s in ("sd_t_d2_fusion_", "sd_t_d2_fusion_host_", "cogent_run", "cogent_%s_run" % e["name"],
+        for s in ("sd_t_d2_fusion_", "sd_t_d2_fusion_host_", "cogent_run", "cogent_run_noalloc", "cogent_%s_run" % e["name"],
                   "cogent_num_indices", "cogent_last_error", "cogent_last_kernel", "cogent_expression", "cogent_info"):
             assert s in syms, (e["name"], s)
 
