@@ -207,6 +207,11 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     # the streaming kernel reads and writes every element of C once, far apart in time: non-temporal C accesses
     # pay there on many shapes whose rows are not whole lines (where the per-tile kernel loses with them)
     specs += [sp + ";nt=3" for sp in specs if "st=" in sp and "nt=" not in sp]
+    # ... with the runs of the workgroups interleaved, so that the tiles in flight chip-wide are neighbours (2 to 6 %
+    # on the shapes with the X panel resident, a loss on some with the Y panel), and with all but the first slice of
+    # the panel loaded behind the first tile (4 % where the panel is a gather of short pieces, nothing elsewhere)
+    specs += [sp + ";il=1" for sp in specs if "st=" in sp and "nt=3" in sp and "il=" not in sp]
+    specs += [sp + ";ov=1" for sp in specs if "st=" in sp and "il=1" in sp and "sy=" not in sp and "ov=" not in sp]
     # the C tile staged through LDS in memory order (every C access a whole line), alone and with non-temporal
     # accesses: pays on HBM-bound shapes whose C rows are not whole lines, most on small tiles
     for sp in [s_ for s_ in extra_specs if "cl=" not in s_][:2] + [c["spec"] for c in cands[:4]]:

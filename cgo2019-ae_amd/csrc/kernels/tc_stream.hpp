@@ -32,6 +32,13 @@
 
 namespace cogent {
 
+// Measurement builds only (never defined by the emitter or the build script): switches parts of the kernel off so
+// that the cost of each can be read from the clock; the results are then wrong.
+// bit 0: no C reads, bit 1: no C writes, bit 2: no loads of the streamed slices, bit 3: no matrix instructions
+#ifndef TC_STREAM_ABLATE
+#define TC_STREAM_ABLATE 0
+#endif
+
 struct TcStreamDims {
     unsigned nres;     // tiles of the whole output along the resident side
     unsigned nstr;     // ... along the streamed side
@@ -93,6 +100,7 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
     constexpr bool NEG_R = (RES == 1) && (Cfg::SIGN < 0);      // "-=" negates the Y operand while it is staged
     constexpr bool NEG_S = (RES == 0) && (Cfg::SIGN < 0);
     constexpr bool VEC4 = SWP;
+    constexpr bool SOV = Cfg::SOV != 0;            // the panel's later slices are loaded behind the first tile
     constexpr bool NT_LD = (Cfg::NTC & 1) != 0, NT_ST = (Cfg::NTC & 2) != 0;
     typedef T T4 __attribute__((ext_vector_type(4)));
 
@@ -116,8 +124,16 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
         vb = xcd * q + (xcd < r ? xcd : r) + idx;
     }
     const unsigned rt = vb % s.nres, rn = vb / s.nres;
-    unsigned st = rn * s.run;
-    const unsigned ntiles = (s.nstr - st) < s.run ? (s.nstr - st) : s.run;
+    // The run of workgroup rn: ntiles streamed-side tiles, `step` apart.  Contiguous runs (SIL = 0): tiles rn * run,
+    // rn * run + 1, ..  Interleaved runs (SIL = 1): tiles rn, rn + nruns, rn + 2 nruns, ..; at any moment the
+    // workgroups are then on NEIGHBOURING tiles, so what is in flight chip-wide is one compact window of C moving
+    // through the tensor instead of nruns windows scattered over it (a bare read-modify-write of the 72^4 fp64
+    // output in these tiles: 4 % faster; the kernels with the X panel resident gain 2 to 6 %, the fp32 shapes with
+    // the Y panel resident lose 5 %, hence an option).
+    constexpr bool SIL = Cfg::SIL != 0;
+    const unsigned step = SIL ? s.nruns : 1u;
+    unsigned st = SIL ? rn : rn * s.run;
+    const unsigned ntiles = SIL ? (s.nstr - rn + s.nruns - 1) / s.nruns : ((s.nstr - st) < s.run ? (s.nstr - st) : s.run);
     // origin of a tile along one side: offset inside C and inside that side's operand
     auto side_origin = [&](auto side_t, unsigned t, int64_t& oc, int64_t& oo) {
         constexpr int SIDE = decltype(side_t)::value;
@@ -152,10 +168,19 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
     // padded tiles: the accumulator elements that fall into the padding have no place in C
     auto c_ok = [&](int ti, int tj, int r) -> bool { return !PADDED || (cx[tj][SWP ? r : 0] >= 0 && cy[ti][SWP ? 0 : r] >= 0); };
 
-    Acc cpre[TY][TX];       // the C tile that the next first K block starts from
+    // CD: how many tiles ahead C is read.  cpre[t % CD] holds the C tile that tile t's first K block starts from;
+    // once that block has taken it, the same registers receive the C tile of tile t + CD.  With CD = 2 a C read has
+    // a whole tile time plus its own to arrive before anything waits for it.
+    constexpr int CD = Cfg::SCD;
+    static_assert(CD == 1 || CD == 2, "C is read one or two tiles ahead");
+    Acc cpre_all[CD][TY][TX];
     Acc acc[TY][TX];
-    auto c_read = [&](const T* base, int ti, int tj) {
-        if (VEC4) {
+    auto c_read = [&](auto par_t, const T* base, int ti, int tj) {
+        Acc (&cpre)[TY][TX] = cpre_all[decltype(par_t)::value];
+        if (TC_STREAM_ABLATE & 1) {
+#pragma unroll
+            for (int r = 0; r < NREG; r++) cpre[ti][tj][r] = (T)0;
+        } else if (VEC4) {
 #pragma unroll
             for (int g = 0; g < NREG / 4; g++) {
                 T4 v = {(T)0, (T)0, (T)0, (T)0};
@@ -173,7 +198,11 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
         }
     };
     auto c_write = [&](T* base, int ti, int tj) {
-        if (VEC4) {
+        if (TC_STREAM_ABLATE & 2) {
+            // keep the accumulators alive without a store
+#pragma unroll
+            for (int r = 0; r < NREG; r++) asm volatile("" :: "v"(acc[ti][tj][r]));
+        } else if (VEC4) {
 #pragma unroll
             for (int g = 0; g < NREG / 4; g++) {
                 T4 v;
@@ -197,25 +226,44 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
     int64_t oc, oo;
     side_origin(str_side, st, oc, oo);
     T* Cb = C + uniform64(baseCr + oc);
+    T* C1 = Cb;                   // CD == 2: the tile after the current one
+    if (CD == 2 && ntiles > 1) {
+        int64_t oc1, oo1;
+        side_origin(str_side, st + step, oc1, oo1);
+        C1 = C + uniform64(baseCr + oc1);
+    }
     const T* const Rsrc = (RES == 0 ? X : Y) + uniform64(baseR);
     const T* const Ssrc = (RES == 0 ? Y : X);
     const T* Sb = Ssrc + uniform64(oo);
     KWalk<Cfg, 1 - RES> ks;       // the K block of the next slice to request
     ks.reset();
     T rs[PD][SLOTS_S];
+    auto s_load = [&](T (&reg)[SLOTS_S], const T* src) {
+        if (TC_STREAM_ABLATE & 4) {
+#pragma unroll
+            for (int i = 0; i < SLOTS_S; i++) reg[i] = (T)(tid + i);
+        } else {
+            slice_load<Cfg, OS, true, true>(reg, src, d, nullptr, tid);
+        }
+    };
     {
         // The panel in groups of RG slices, all loads of a group in flight together (the accumulators
         // are not live yet, so the registers are there).  The requests for the first slices of the stream
         // and for the first C tile follow the last group's: loads return in order, and the panel and the
         // slices come from L2 while C comes from HBM.
         constexpr int RREG = SLOTS_R * (int)sizeof(T) / 4;
-        constexpr int RG = (NKB * RREG <= 96) ? NKB : (96 / RREG < 1 ? 1 : 96 / RREG);
-        constexpr int NG = (NKB + RG - 1) / RG;
+        // SOV: only the panel's FIRST slice is loaded here; slice j + 1 is requested during trip j of the first
+        // tile, which needs no more than slice j of the panel.  The gather of a panel whose memory order does not
+        // match the tile (16-byte pieces of distinct lines) is bound by the L2, not by HBM: behind the first tile's
+        // C traffic it costs nothing, in front of it the whole chip waits.
+        constexpr int NPRO = SOV ? 1 : NKB;
+        constexpr int RG = (NPRO * RREG <= 96) ? NPRO : (96 / RREG < 1 ? 1 : 96 / RREG);
+        constexpr int NG = (NPRO + RG - 1) / RG;
         KWalk<Cfg, RES> kr;
         kr.reset();
         static_for<NG>([&](auto gt) {
             constexpr int j0 = decltype(gt)::value * RG;
-            constexpr int n = (NKB - j0) < RG ? (NKB - j0) : RG;
+            constexpr int n = (NPRO - j0) < RG ? (NPRO - j0) : RG;
             T rr[n][SLOTS_R];
             static_for<n>([&](auto it) {
                 slice_load<Cfg, OR, true, true>(rr[decltype(it)::value], Rsrc + uniform64(kr.offset(d)), d, nullptr, tid);
@@ -223,13 +271,19 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
             });
             if constexpr (decltype(gt)::value == NG - 1) {
                 static_for<PD>([&](auto sg) {
-                    slice_load<Cfg, OS, true, true>(rs[decltype(sg)::value], Sb + uniform64(ks.offset(d)), d, nullptr, tid);
+                    s_load(rs[decltype(sg)::value], Sb + uniform64(ks.offset(d)));
                     ks.next(d);
                 });
 #pragma unroll
                 for (int ti = 0; ti < TY; ti++)
 #pragma unroll
-                    for (int tj = 0; tj < TX; tj++) c_read(Cb, ti, tj);
+                    for (int tj = 0; tj < TX; tj++) c_read(std::integral_constant<int, 0>(), Cb, ti, tj);
+                if (CD == 2) {            // (a run of a single tile reads its own C a second time: no branch here)
+#pragma unroll
+                    for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+                        for (int tj = 0; tj < TX; tj++) c_read(std::integral_constant<int, CD - 1>(), C1, ti, tj);
+                }
             }
             static_for<n>([&](auto it) {
                 slice_store<Cfg, OR, NEG_R, VR>(rr[decltype(it)::value], lds_r + (j0 + decltype(it)::value) * LDS_R, d, tid);
@@ -242,30 +296,53 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
 
     // ---- one output tile: NKB trips.  Slice j of the tile is in LDS stage (sbuf + j) % 2 when trip j
     // starts; register stage j % PD is free then and takes the request for slice j + PD of the stream.
-    auto tile = [&](auto has_next_t) {
+    KWalk<Cfg, RES> kp;           // SOV: the panel slice to request next (slice 0 came with the prologue)
+    kp.reset();
+    kp.next(d);
+    // PAR = t % CD; HAS_NEXT: tile t + 1 exists (its slices are requested here); HAS_FAR: tile t + CD exists (its C
+    // is read here); FIRST: tile 0
+    auto tile = [&](auto par_t, auto has_next_t, auto has_far_t, auto first_t) {
         constexpr bool HAS_NEXT = decltype(has_next_t)::value;
-        T* Cn = Cb;
+        constexpr bool HAS_FAR = decltype(has_far_t)::value;
+        constexpr bool FIRST = SOV && decltype(first_t)::value;
+        Acc (&cpre)[TY][TX] = cpre_all[decltype(par_t)::value];
+        T* Cf = Cb;
         const T* Sn = Sb;
         if (HAS_NEXT) {
-            side_origin(str_side, st + 1, oc, oo);
-            Cn = C + uniform64(baseCr + oc);
+            side_origin(str_side, st + step, oc, oo);
             Sn = Ssrc + uniform64(oo);
+            if (CD == 1) Cf = C + uniform64(baseCr + oc);
+        }
+        if (CD == 2 && HAS_FAR) {
+            int64_t ocf, oof;
+            side_origin(str_side, st + 2 * step, ocf, oof);
+            Cf = C + uniform64(baseCr + ocf);
         }
         static_for<NKB>([&](auto jt) {
             constexpr int j = decltype(jt)::value;
             constexpr int S = j % PD;
+            // first tile, SOV: the panel's slice j + 1, requested before anything else of this trip so that the
+            // wait for it at the end of the trip (loads return in order) leaves the younger requests in flight
+            constexpr bool PANEL = FIRST && (j + 1 < NKB);
+            T rp[PANEL ? SLOTS_R : 1];
+            if constexpr (PANEL) {
+                slice_load<Cfg, OR, true, true>(rp, Rsrc + uniform64(kp.offset(d)), d, nullptr, tid);
+                kp.next(d);
+            }
             if constexpr (j + PD < NKB) {
-                slice_load<Cfg, OS, true, true>(rs[S], Sb + uniform64(ks.offset(d)), d, nullptr, tid);
+                s_load(rs[S], Sb + uniform64(ks.offset(d)));
                 ks.next(d);
             } else if constexpr (HAS_NEXT) {
-                slice_load<Cfg, OS, true, true>(rs[S], Sn + uniform64(ks.offset(d)), d, nullptr, tid);
+                s_load(rs[S], Sn + uniform64(ks.offset(d)));
                 ks.next(d);
             }
-            // the next tile's C, spread over trips 1 .. NKB-1 (trip 0 still reads these registers)
-            if constexpr (HAS_NEXT && j >= 1) {
+            // the C of tile t + CD, spread over trips 1 .. NKB-1: trip 0's first matrix step still reads these registers.
+            // (Requesting it earlier -- from trip 0 on, or all of it right after that first step -- measured 3 to 10 %
+            // slower on the 72^5 fp64 shape, all of it in the last trip 4 % slower.)
+            if constexpr (HAS_FAR && j >= 1) {
                 static_for<TY * TX>([&](auto ct) {
                     constexpr int c = decltype(ct)::value;
-                    if constexpr (1 + (c * (NKB - 1)) / (TY * TX) == j) c_read(Cn, c / TX, c % TX);
+                    if constexpr (1 + (c * (NKB - 1)) / (TY * TX) == j) c_read(par_t, Cf, c / TX, c % TX);
                 });
             }
             const T* lr = lds_r + j * LDS_R;
@@ -285,9 +362,11 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
 #pragma unroll
                     for (int tj = 0; tj < TX; tj++) {
                         const Acc from = (j == 0 && k4 == 0) ? cpre[ti][tj] : acc[ti][tj];
-                        acc[ti][tj] = SWP ? MM::mma(b[tj], a[ti], from) : MM::mma(a[ti], b[tj], from);
+                        if (TC_STREAM_ABLATE & 8) { asm volatile("" :: "v"(a[ti]), "v"(b[tj])); acc[ti][tj] = from; }
+                        else acc[ti][tj] = SWP ? MM::mma(b[tj], a[ti], from) : MM::mma(a[ti], b[tj], from);
                     }
             }
+            if constexpr (PANEL) slice_store<Cfg, OR, NEG_R, VR>(rp, lds_r + (j + 1) * LDS_R, d, tid);
             if constexpr (j + 1 < NKB || HAS_NEXT) {
                 T* dst = lds_s + (NKB % 2 == 0 ? ((j + 1) & 1) : (sbuf ^ ((j + 1) & 1))) * LDS_S;
                 slice_store<Cfg, OS, NEG_S, VS>(rs[(j + 1) % PD], dst, d, tid);
@@ -299,18 +378,39 @@ void tc_stream_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __
 #pragma unroll
             for (int tj = 0; tj < TX; tj++) c_write(Cb, ti, tj);
         if (HAS_NEXT) {
-            Cb = Cn; Sb = Sn; st++;
+            Cb = (CD == 1) ? Cf : C1;
+            C1 = Cf;
+            Sb = Sn; st += step;
             if (NKB % 2) sbuf ^= 1;
         }
     };
 
     // The first tile is a copy of its own so that the tiles inside the loop all start from the same
     // history of loads and stores in flight; the last tile requests nothing further.
-    if (ntiles > 1) {
-        tile(std::true_type());
-        for (unsigned t = 2; t < ntiles; t++) tile(std::true_type());
+    const std::integral_constant<int, 0> P0;
+    const std::integral_constant<int, CD - 1> P1;       // parity 1 (CD == 1: the one register tile)
+    const std::true_type yes;
+    const std::false_type no;
+    if (CD == 1) {
+        if (ntiles > 1) {
+            if (SOV) tile(P0, yes, yes, yes); else tile(P0, yes, yes, no);
+            for (unsigned t = 2; t < ntiles; t++) tile(P0, yes, yes, no);
+            tile(P0, no, no, no);
+        } else {
+            if (SOV) tile(P0, no, no, yes); else tile(P0, no, no, no);
+        }
+    } else {
+        // tile 0, then pairs (odd, even) while at least four tiles remain, then the last one to three tiles
+        unsigned left = ntiles;
+        if (left >= 3)      { if (SOV) tile(P0, yes, yes, yes); else tile(P0, yes, yes, no); }
+        else if (left == 2) { if (SOV) tile(P0, yes, no, yes); else tile(P0, yes, no, no); }
+        else                { if (SOV) tile(P0, no, no, yes); else tile(P0, no, no, no); }
+        left--;
+        for (; left >= 4; left -= 2) { tile(P1, yes, yes, no); tile(P0, yes, yes, no); }
+        if (left == 3)      { tile(P1, yes, yes, no); tile(P0, yes, no, no); tile(P1, no, no, no); }
+        else if (left == 2) { tile(P1, yes, no, no); tile(P0, no, no, no); }
+        else if (left == 1) { tile(P1, no, no, no); }
     }
-    tile(std::false_type());
 }
 
 }  // namespace cogent

@@ -93,7 +93,8 @@ void emit_cfg_members(std::ostringstream& o, const Contraction& c, DType t, cons
         // elements per slice load: as many as 16 bytes hold, when the tile of the operand's fastest index is a multiple
         const int vmax = (t == DType::F64) ? 2 : 4;
         const int t0 = tiles.empty() ? 1 : tiles[0];
-        const int vw = !m.VL ? 1 : (t0 % vmax == 0 ? vmax : (t0 % 2 == 0 ? 2 : 1));
+        const bool on = m.VL == 1 || (m.VL == 2 && p[0] == 'X') || (m.VL == 3 && p[0] == 'Y');      // vl=1 both inputs, 2 the X side only, 3 the Y side only
+        const int vw = !on ? 1 : (t0 % vmax == 0 ? vmax : (t0 % 2 == 0 ? 2 : 1));
         o << "    static constexpr int VW" << p << " = " << vw << ";\n";
         std::string s(1, (char)tolower(p[0]));
         o << table((s + "o_id").c_str(), ids) << table((s + "o_tile").c_str(), tiles)
@@ -104,7 +105,7 @@ void emit_cfg_members(std::ostringstream& o, const Contraction& c, DType t, cons
     operand("Y", yop, m.y_ids, m.y_tiles);
     o << "    static constexpr int WX = " << m.WX << ", WY = " << m.WY << ", TX = " << m.TX << ", TY = " << m.TY << ", NT = " << 64 * m.WX * m.WY << ";\n";
     o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", SKO = " << m.SKO << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ", RPX = " << m.RPX << ", RPY = " << m.RPY << ", CLDS = " << m.CLDS << ", NTO = " << m.NTO << ";\n";
-    o << "    static constexpr int STREAM = " << m.STREAM << ", SPD = " << m.SPD << ", SMW = " << m.SMW << ", SRES = " << m.SRES << ", DBUF = " << m.DBUF << ";\n";
+    o << "    static constexpr int STREAM = " << m.STREAM << ", SPD = " << m.SPD << ", SMW = " << m.SMW << ", SRES = " << m.SRES << ", SOV = " << m.SOV << ", SCD = " << m.SCD << ", SIL = " << m.SIL << ", DBUF = " << m.DBUF << ";\n";
     o << "    static constexpr int LAYX = " << m.layx << ", LDX = " << m.ldx << ", LAYY = " << m.layy << ", LDY = " << m.ldy << ";\n";
 }
 

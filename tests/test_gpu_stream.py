@@ -17,7 +17,9 @@ TOL = {"f64": 1e-12, "f32": 1e-5}
 STREAMING = ["cfg2_f64", "var_cfg2_stream96_f64", "var_cfg4_stream_f32", "var_stream_2k_f64",
              "var_tccg11_stream_y_f64",      # the Y panel resident, its 72 rows padded to 80
              "var_tccg09_stream_pad_f64",    # the X panel resident, its 72 columns padded to 80
-             "var_cfg4_stream_pad_f32"]      # fp32, 128-bit C accesses, a Y tile of 24 rows padded to 32
+             "var_cfg4_stream_pad_f32",      # fp32, 128-bit C accesses, a Y tile of 24 rows padded to 32
+             "var_cfg2_stream_cd2_f64",      # C read two tiles ahead (runs of 12 and 9 tiles: both parities end a run)
+             "var_tccg11_stream_y_ov_f64"]   # Y panel loaded behind the first tile, interleaved runs, C two tiles ahead
 
 
 def _check(name, sizes, tools, oracle, variant=None, expect=None):
@@ -47,7 +49,7 @@ def test_objects_carry_the_streaming_kernel(name):
     info = pkg.Expression(name).info
     nkb, depth = info["stream"]
     assert nkb >= 2 and depth >= 1 and nkb % depth == 0
-    assert info["stream_resident"] == ("y" if name == "var_tccg11_stream_y_f64" else "x")
+    assert info["stream_resident"] == ("y" if name.startswith("var_tccg11_stream_y") else "x")
 
 
 @pytest.mark.parametrize("name", STREAMING)

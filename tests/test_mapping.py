@@ -150,6 +150,12 @@ def test_streaming_kernel_option(tools, tmp_path):
     assert m["stream_resident"] == "x"
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:8,a:8;k=e:24;w=3x4;t=3x1;st=3;sy=1").info["mapping"]
     assert m["stream_resident"] == "y" and "sy=1" in m["spec"]
+    # the streaming kernel's own options round-trip through the spec: interleaved runs, the panel behind the first
+    # tile, C read two tiles ahead; 16-byte slice loads per side
+    m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:8,a:8;k=e:24;w=3x4;t=3x1;st=3;il=1;ov=1;cd=2;vl=2").info["mapping"]
+    assert (m["stream_interleaved_runs"], m["stream_panel_overlap"], m["stream_c_distance"], m["vector_slice_loads"]) == (1, 1, 2, 2)
+    assert all(k in m["spec"] for k in ("il=1", "ov=1", "cd=2", "vl=2"))
+    assert tools.plan(text, "DOUBLE", mapping_spec=m["spec"]).info["mapping"] == m
     # tiles padded to the MFMA granularity are allowed (a 72-wide side runs as 80)
     text9 = open(os.path.join(EXPR_DIR, "tccg_09.in")).read()
     m = tools.plan(text9, "DOUBLE", mapping_spec="x=a:72;y=b:8,c:8,d:1;k=e:24;w=1x4;t=5x1;st=3").info["mapping"]
