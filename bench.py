@@ -31,7 +31,8 @@ HEADLINE = "cfg2_f64"
 
 
 def read_traffic(name):
-    """HBM bytes per launch from the rocprofv3 counter summary under profiles/, or None."""
+    """HBM bytes per launch from the rocprofv3 counter summary under profiles/ (FETCH_SIZE and WRITE_SIZE of the
+    contraction kernel, each scaled by what the same counter reads for a plain copy of known size), or None."""
     path = os.path.join(ROOT, "profiles", "traffic_%s.txt" % name)
     if not os.path.exists(path):
         return None
@@ -41,11 +42,23 @@ def read_traffic(name):
     return None
 
 
+def read_mfma_busy(name):
+    """Fraction of the kernel's active cycles with the matrix cores busy, from the counter summary under profiles/, or None."""
+    path = os.path.join(ROOT, "profiles", "mfma_%s.txt" % name)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("mfma_busy_fraction:"):
+            return float(line.split(":")[1])
+    return None
+
+
 class Workload:
     def __init__(self, pkg, tools, entry, sizes):
         import numpy as np
         import torch
         self.name = entry["name"]
+        self.plan_file = entry["file"]
         self.sizes = list(sizes)
         self.ex = pkg.Expression(self.name)
         self.plan = tools.plan(pkg.expression_text(self.name), entry["dtype"])
@@ -107,60 +120,71 @@ def time_workload(driver, w, warmup, iters, min_warm_ms=30.0):
     warmup = len(w.dC) + int(min(2000, max(0.0, min_warm_ms / max(probe["mean_ms"], 1e-3) - warmup)))
     st = driver.time(w.ex, w.sizes, w.c_ptrs(), w.dA.data_ptr(), w.dB.data_ptr(), warmup, iters)
     primary, secondary = roofline(w, st["mean_ms"])
-    return {"name": w.name, "sizes": w.sizes, "dtype": w.dtype, "flops": w.flops, "algorithmic_bytes": w.bytes,
-            "kernel_us_mean": round(st["mean_ms"] * 1e3, 2), "kernel_us_median": round(st["median_ms"] * 1e3, 2),
-            "kernel_us_min": round(st["min_ms"] * 1e3, 2),
-            "gflops": round(w.flops / (st["mean_ms"] * 1e-3) / 1e9, 1),
-            "roofline": primary, "roofline_other": secondary,
-            "mapping": w.ex.info["spec"]}
+    for r in (primary, secondary):
+        if r["bound"] == "hbm":
+            r["traffic"] = read_traffic(w.name)
+        elif read_mfma_busy(w.name) is not None:
+            r["mfma_busy_fraction_rocprof"] = read_mfma_busy(w.name)
+    row = {"name": w.name, "sizes": w.sizes, "dtype": w.dtype, "flops": w.flops, "algorithmic_bytes": w.bytes,
+           "kernel_us_mean": round(st["mean_ms"] * 1e3, 2), "kernel_us_median": round(st["median_ms"] * 1e3, 2),
+           "kernel_us_min": round(st["min_ms"] * 1e3, 2),
+           "gflops": round(w.flops / (st["mean_ms"] * 1e-3) / 1e9, 1),
+           "roofline": primary, "roofline_other": secondary,
+           "mapping": w.ex.info["spec"], "kernel": w.ex.last_kernel()}
+    if primary["bound"] == "hbm" and 2 * w.nC * (8 if w.dtype == "f64" else 4) > 0.5 * w.bytes:
+        # the same output tensor read, incremented and written back by a bare streaming kernel (non-temporal, 8 loads
+        # in flight per lane) on the same rotated buffers: what the memory system gives the C traffic alone
+        esize = 8 if w.dtype == "f64" else 4
+        ms = driver.time_rmw(w.c_ptrs(), w.nC * esize, 1, 20, 50)
+        row["c_rmw_stream_us"] = round(ms * 1e3, 2)
+        row["c_rmw_stream_GBps"] = round(2 * w.nC * esize / ms / 1e6, 1)
+        w.reset_c()
+    return row
 
 
-def cpu_baseline_and_verify(w, budget_s=20.0):
-    """Times the CPU oracle on a slab of the output (whole tensor when it fits the time budget) and
-    checks the GPU result on that slab.  Runs after ONE launch from a fresh C."""
+def cpu_baseline_and_verify(w, one_thread=False, repeat_s=1.0):
+    """The CPU oracle (the reference's host nested-loop contraction, cogent/drivers/tccg/code_main_tccg_01.c:117-133)
+    computes the WHOLE contraction on this box's cores: timed (median of a few runs when one takes under repeat_s
+    seconds) and used to check EVERY element of one GPU launch from a fresh C.  one_thread: also one run on a single thread."""
     import numpy as np
     import torch
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import helpers
     oracle = helpers.Oracle()
-    pkg_text = open(os.path.join(ROOT, "cgo2019-ae_amd", "expressions", w.plan_file)).read()
-    expr = helpers.parse_expression(pkg_text)
+    expr = helpers.parse_expression(open(os.path.join(ROOT, "cgo2019-ae_amd", "expressions", w.plan_file)).read())
     threads = min(oracle.max_threads(), 16)
-    last = w.sizes[len(expr["out_idx"]) - 1]
-    # probe one slice of the slowest output index to size the sample
-    probe = w.hC.copy()
-    t0 = time.perf_counter()
-    oracle.contract(expr, w.sizes, probe, w.hA, w.hB, threads=threads, last_range=(0, 1))
-    per_slice = time.perf_counter() - t0
-    n_slices = int(max(1, min(last, budget_s / max(per_slice, 1e-6))))
     want = w.hC.copy()
-    t0 = time.perf_counter()
-    oracle.contract(expr, w.sizes, want, w.hA, w.hB, threads=threads, last_range=(0, n_slices))
-    cpu_s = time.perf_counter() - t0
-    # a short sample is noisy (thread start-up, a busy host): repeat it for about five seconds, keep the median
-    runs = [cpu_s]
-    scratch = w.hC.copy()
-    while sum(runs) < min(budget_s, 5.0) and len(runs) < 50:
-        np.copyto(scratch, w.hC)
+    runs = []
+    while True:
+        np.copyto(want, w.hC)
         t0 = time.perf_counter()
-        oracle.contract(expr, w.sizes, scratch, w.hA, w.hB, threads=threads, last_range=(0, n_slices))
+        oracle.contract(expr, w.sizes, want, w.hA, w.hB, threads=threads)
         runs.append(time.perf_counter() - t0)
+        if sum(runs) >= repeat_s or len(runs) >= 9:
+            break
     cpu_s = sorted(runs)[len(runs) // 2]
-    frac = n_slices / last
-    slab = (w.nC // last) * n_slices
-    # one GPU launch from a fresh C
+    base = {"value": round(w.flops / cpu_s / 1e9, 2), "unit": "GFLOP/s", "cores": threads, "kind": "port",
+            "sample": "the whole contraction (%d flop), median of %d run(s), %.3f s each on %d threads" % (w.flops, len(runs), cpu_s, threads)}
+    if one_thread:
+        scratch = w.hC.copy()
+        t0 = time.perf_counter()
+        oracle.contract(expr, w.sizes, scratch, w.hA, w.hB, threads=1)
+        t1 = time.perf_counter() - t0
+        base["one_thread"] = {"value": round(w.flops / t1 / 1e9, 2), "unit": "GFLOP/s", "cores": 1, "seconds": round(t1, 3),
+                              "identical_to_all_threads": bool(np.array_equal(scratch, want))}
+    # one GPU launch from a fresh C, every element compared
     w.reset_c()
     w.launch(0)
     torch.cuda.synchronize()
     got = w.dC[0].cpu().numpy()
-    err = helpers.rel_error(got[:slab], want[:slab])
+    err = helpers.rel_error(got, want)
     w.reset_c()
-    base = {"value": round(w.flops * frac / cpu_s / 1e9, 2), "unit": "GFLOP/s", "cores": threads, "kind": "port",
-            "sample": "%d of %d slices of the slowest output index (%.0f%% of the contraction), median of %d runs, %.2f s wall each on %d threads"
-                      % (n_slices, last, 100 * frac, len(runs), cpu_s, threads)}
-    verify = {"checked_elements": int(slab), "max_rel_err": err, "tolerance": TOL[w.dtype],
-              "definition": "|gpu-ref| / max(|ref|, rms(ref))", "pass": bool(err <= TOL[w.dtype])}
+    verify = {"checked_elements": int(want.size), "of_elements": int(w.nC), "max_rel_err": err, "max_abs_err": float(np.max(np.abs(got.astype(np.float64) - want))),
+              "tolerance": TOL[w.dtype], "definition": "|gpu-ref| / max(|ref|, rms(ref))", "pass": bool(err <= TOL[w.dtype])}
     return base, verify
+
+
+ONE_THREAD = ("cfg1_", "cfg2_", "cfg4_16_", "cfg5_")      # the configs a single-thread CPU figure is reported for
 
 
 def main():
@@ -173,6 +197,9 @@ def main():
     ap.add_argument("--workload", default=HEADLINE, help="expression object to use as the headline workload")
     ap.add_argument("--suite", default="", help="'fused': time the fused groups of the manifest; 'tccg': time the 48 TCCG contractions at the sizes of the reference's "
                     "bench script (cogent/bench_tccg.sh:5-54) and print one JSON line with the table, instead of the headline run")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="only run the memory yardsticks: plain copy and bare read-modify-write streams (flat, and in the streaming "
+                         "kernel's tiles of config 2's output) at the output sizes of the HBM-bound configs; one JSON line")
     ap.add_argument("--copy-only", type=int, default=0, metavar="BYTES",
                     help="only run the plain device-to-device copy kernel on BYTES bytes, --steps times "
                          "(the known-size yardstick the FETCH_SIZE / WRITE_SIZE counter readings are scaled by)")
@@ -196,6 +223,26 @@ def main():
         ms = driver.time_copy(src.data_ptr(), dst.data_ptr(), args.copy_only, args.warmup, args.steps)
         print(json.dumps({"copy_bytes": args.copy_only, "ms_per_copy": ms,
                           "GBps_read_plus_write": round(2 * args.copy_only / ms / 1e6, 1)}))
+        return
+
+    if args.ceilings:
+        rows = []
+        for label, nbytes in (("C4-16 output (fp32 16^6)", 4 * 16 ** 6), ("C5 output (fp64 16^6)", 8 * 16 ** 6),
+                              ("C2 output (fp64 72^4)", 8 * 72 ** 4), ("C4-24 output (fp32 24^6)", 4 * 24 ** 6)):
+            n_rot = max(2, min(8, int(1.2e9 // nbytes) + 1))
+            bufs = [torch.zeros(nbytes // 8, dtype=torch.float64, device="cuda") for _ in range(n_rot)]
+            ptrs = [b.data_ptr() for b in bufs]
+            row = {"what": label, "bytes": nbytes, "buffers_rotated": n_rot}
+            for mode, key in ((0, "rmw_flat"), (1, "rmw_flat_nontemporal")) + (((2, "rmw_stream_kernel_tiles"), (3, "rmw_stream_kernel_tiles_interleaved")) if nbytes == 8 * 72 ** 4 else ()):
+                ms = min(driver.time_rmw(ptrs, nbytes, mode, 30, max(20, args.steps)) for _ in range(3))
+                row[key] = {"us": round(ms * 1e3, 2), "GBps_read_plus_write": round(2 * nbytes / ms / 1e6, 1), "frac_of_8TBps": round(2 * nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            ms = driver.time_copy(bufs[0].data_ptr(), bufs[1].data_ptr(), nbytes, 30, max(20, args.steps))
+            row["copy"] = {"us": round(ms * 1e3, 2), "GBps_read_plus_write": round(2 * nbytes / ms / 1e6, 1)}
+            rows.append(row)
+            print("%-28s %s" % (label, {k: v["us"] for k, v in row.items() if isinstance(v, dict)}), file=sys.stderr, flush=True)
+            del bufs
+            torch.cuda.empty_cache()
+        print(json.dumps({"ceilings": rows, "unit": "us per launch, mean over back-to-back launches on rotated buffers", "hbm_peak_GBps": HBM_PEAK_GBS}))
         return
 
     if args.suite == "fused":
@@ -257,11 +304,10 @@ def main():
 
     entry = pkg.manifest_entry(args.workload)
     w = Workload(pkg, tools, entry, entry["bench_sizes"])
-    w.plan_file = entry["file"]
 
     cpu, verify = (None, None)
     if not args.no_cpu:
-        cpu, verify = cpu_baseline_and_verify(w)
+        cpu, verify = cpu_baseline_and_verify(w, one_thread=w.name.startswith(ONE_THREAD), repeat_s=5.0)
 
     # ---- the timed region: W warm-up steps, then exactly K steps between two synchronisations
     for i in range(args.warmup):
@@ -276,7 +322,7 @@ def main():
 
     # ---- per-launch kernel durations from HIP events on the launch stream
     head = time_workload(driver, w, args.warmup, args.steps)
-    head["roofline"]["traffic"] = read_traffic(w.name)
+    head["roofline"].setdefault("traffic", read_traffic(w.name))
 
     table = []
     if not args.only_headline:
@@ -287,7 +333,12 @@ def main():
                 continue
             for sizes in [e["bench_sizes"]] + e.get("alt_sizes", []):
                 wl = Workload(pkg, tools, e, sizes)
-                table.append(time_workload(driver, wl, 10, 50))
+                row = time_workload(driver, wl, 10, 50)
+                if not args.no_cpu:
+                    row["cpu_baseline"], row["verify"] = cpu_baseline_and_verify(wl, one_thread=wl.name.startswith(ONE_THREAD))
+                table.append(row)
+                print("%-12s %-28s %8.1f us  %s %.3f  verify %s" % (row["name"], row["sizes"], row["kernel_us_mean"], row["roofline"]["bound"],
+                      row["roofline"]["frac"], row.get("verify", {}).get("pass")), file=sys.stderr, flush=True)
                 del wl
                 torch.cuda.empty_cache()
 

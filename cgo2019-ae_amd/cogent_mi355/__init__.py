@@ -269,6 +269,9 @@ class Driver:
         lib.cogent_driver_time_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int,
                                                 ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
         lib.cogent_driver_time_copy.restype = ctypes.c_int
+        lib.cogent_driver_time_rmw.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_longlong, ctypes.c_int,
+                                               ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+        lib.cogent_driver_time_rmw.restype = ctypes.c_int
         lib.cogent_driver_last_error.restype = ctypes.c_char_p
         self.lib = lib
 
@@ -299,6 +302,16 @@ class Driver:
         if rc:
             raise CogentError("timing failed (%d): %s" % (rc, self.lib.cogent_driver_last_error().decode()))
         return {"mean_ms": stats[0], "median_ms": stats[1], "min_ms": stats[2], "max_ms": stats[3], "each_ms": list(each)}
+
+    def time_rmw(self, buf_ptrs, nbytes, mode, warmup, iters):
+        """Mean ms per launch of a bare read-modify-write of nbytes: mode 0 flat, 1 flat non-temporal, 2 / 3 in the tiles of the
+        streaming kernel on config 2's output (contiguous / interleaved runs)."""
+        bufs = (ctypes.c_void_p * len(buf_ptrs))(*buf_ptrs)
+        stats = (ctypes.c_float * 4)()
+        rc = self.lib.cogent_driver_time_rmw(bufs, len(buf_ptrs), nbytes, mode, warmup, iters, stats)
+        if rc:
+            raise CogentError("read-modify-write timing failed (%d)" % rc)
+        return stats[0]
 
     def time_copy(self, src_ptr, dst_ptr, nbytes, warmup, iters):
         stats = (ctypes.c_float * 4)()
