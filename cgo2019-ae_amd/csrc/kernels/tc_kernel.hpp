@@ -358,53 +358,76 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     int rem[Cfg::NIDX];
     int64_t baseC = 0, baseX = 0, baseY = 0;
     {
-        // Workgroups are handed to the 8 XCDs round-robin and every XCD has its own L2: give XCD x
-        // a CONTIGUOUS range of output tiles, so that the tiles resident on one XCD share their
-        // operand panels in that L2.
-        unsigned b;
-        {
-            const unsigned n = d.nblocks, xcd = blockIdx.x % 8u, idx = blockIdx.x / 8u;
-            const unsigned q = n / 8u, r = n % 8u;
-            b = xcd * q + (xcd < r ? xcd : r) + idx;
-        }
-        // split K: SK consecutive workgroups share one output tile, each takes a share of the K blocks.
-        // SKO: the shares are the outermost level instead, so an XCD's range holds ALL tiles of a few
-        // shares and the operand slices those tiles have in common meet in that XCD's L2.
-        if (SK > 1) {
-            if (Cfg::SKO != 0) { const unsigned nt = d.nblocks / (unsigned)SK; ks = b / nt; b %= nt; }
-            else               { ks = b % (unsigned)SK; b /= (unsigned)SK; }
-        }
-        // Within that range walk the tile grid in bands of TILE_GROUP X-tiles (X fastest inside a
-        // band, then Y): the ~100 tiles in flight on an XCD then touch a dozen X panels and a dozen
-        // Y panels instead of every X panel, and the panels stay in the 4 MB L2 while C streams by.
-        {
-            constexpr unsigned GX = 8;
-            const unsigned nyt = (d.nblocks / (unsigned)SK) / d.nxt;
-            const unsigned G = GX * nyt;
-            const unsigned g = b / G, r = b % G;
-            const unsigned first = g * GX;
-            const unsigned gx = (d.nxt - first) < GX ? (d.nxt - first) : GX;
-            b = (first + r % gx) + (r / gx) * d.nxt;
-        }
+        if constexpr (Cfg::TORD != 0) {
+            // Tile order = the order of the tile origins in C's memory, workgroup b = blockIdx.x: the workgroups in
+            // flight chip-wide (consecutive ones go to different XCDs) then cover ONE compact window of C that moves
+            // linearly through the tensor, the access pattern of a plain streaming kernel.  For outputs much larger
+            // than the inputs (which then sit in every XCD's L2 anyway) this is what the memory system likes best.
+            unsigned b = blockIdx.x;
+            if (SK > 1) {
+                if (Cfg::SKO != 0) { const unsigned nt = d.nblocks / (unsigned)SK; ks = b / nt; b %= nt; }
+                else               { ks = b % (unsigned)SK; b /= (unsigned)SK; }
+            }
 #pragma unroll
-        for (int i = 0; i < Cfg::NX; i++) {
-            const int id = Cfg::x_id(i);
-            const unsigned nb = (unsigned)d.nblk[id];
-            const int o = (int)(b % nb) * Cfg::x_tile(i);
-            b /= nb;
-            rem[id] = d.ext[id] - o;
-            baseC += (int64_t)o * d.sC[id];
-            baseX += (int64_t)o * d.sX[id];
-        }
+            for (int j = 0; j < Cfg::CR; j++) {
+                const int id = Cfg::c_id(j);
+                const unsigned nb = (unsigned)d.nblk[id];
+                const int o = (int)(b % nb) * Cfg::c_tile(j);
+                b /= nb;
+                rem[id] = d.ext[id] - o;
+                baseC += (int64_t)o * d.sC[id];
+                baseX += (int64_t)o * d.sX[id];         // (the stride is zero in the operand that does not hold the index)
+                baseY += (int64_t)o * d.sY[id];
+            }
+        } else {
+            // Workgroups are handed to the 8 XCDs round-robin and every XCD has its own L2: give XCD x
+            // a CONTIGUOUS range of output tiles, so that the tiles resident on one XCD share their
+            // operand panels in that L2.
+            unsigned b;
+            {
+                const unsigned n = d.nblocks, xcd = blockIdx.x % 8u, idx = blockIdx.x / 8u;
+                const unsigned q = n / 8u, r = n % 8u;
+                b = xcd * q + (xcd < r ? xcd : r) + idx;
+            }
+            // split K: SK consecutive workgroups share one output tile, each takes a share of the K blocks.
+            // SKO: the shares are the outermost level instead, so an XCD's range holds ALL tiles of a few
+            // shares and the operand slices those tiles have in common meet in that XCD's L2.
+            if (SK > 1) {
+                if (Cfg::SKO != 0) { const unsigned nt = d.nblocks / (unsigned)SK; ks = b / nt; b %= nt; }
+                else               { ks = b % (unsigned)SK; b /= (unsigned)SK; }
+            }
+            // Within that range walk the tile grid in bands of TILE_GROUP X-tiles (X fastest inside a
+            // band, then Y): the ~100 tiles in flight on an XCD then touch a dozen X panels and a dozen
+            // Y panels instead of every X panel, and the panels stay in the 4 MB L2 while C streams by.
+            {
+                constexpr unsigned GX = 8;
+                const unsigned nyt = (d.nblocks / (unsigned)SK) / d.nxt;
+                const unsigned G = GX * nyt;
+                const unsigned g = b / G, r = b % G;
+                const unsigned first = g * GX;
+                const unsigned gx = (d.nxt - first) < GX ? (d.nxt - first) : GX;
+                b = (first + r % gx) + (r / gx) * d.nxt;
+            }
 #pragma unroll
-        for (int i = 0; i < Cfg::NY; i++) {
-            const int id = Cfg::y_id(i);
-            const unsigned nb = (unsigned)d.nblk[id];
-            const int o = (int)(b % nb) * Cfg::y_tile(i);
-            b /= nb;
-            rem[id] = d.ext[id] - o;
-            baseC += (int64_t)o * d.sC[id];
-            baseY += (int64_t)o * d.sY[id];
+            for (int i = 0; i < Cfg::NX; i++) {
+                const int id = Cfg::x_id(i);
+                const unsigned nb = (unsigned)d.nblk[id];
+                const int o = (int)(b % nb) * Cfg::x_tile(i);
+                b /= nb;
+                rem[id] = d.ext[id] - o;
+                baseC += (int64_t)o * d.sC[id];
+                baseX += (int64_t)o * d.sX[id];
+            }
+#pragma unroll
+            for (int i = 0; i < Cfg::NY; i++) {
+                const int id = Cfg::y_id(i);
+                const unsigned nb = (unsigned)d.nblk[id];
+                const int o = (int)(b % nb) * Cfg::y_tile(i);
+                b /= nb;
+                rem[id] = d.ext[id] - o;
+                baseC += (int64_t)o * d.sC[id];
+                baseY += (int64_t)o * d.sY[id];
+            }
         }
 #pragma unroll
         for (int i = 0; i < Cfg::NK; i++) rem[Cfg::k_id(i)] = d.ext[Cfg::k_id(i)];

@@ -26,6 +26,10 @@
  * with the reference's own compiled loops (oracle/_ref) for 3-D, 4-D, 2-D and
  * 6-D outputs with one and two contracted indices, fp64 and fp32, "+=" and
  * "-=", and with numpy einsum, closed forms and a brute-force Python loop.
+ * The reference has no driver with three or more contracted indices or with
+ * none; those two branches of the loop below are pinned by hand-written loop
+ * nests with the same summation order (bit-exact), by numpy einsum, by the
+ * two-index branch through a unit extent, and by the outer-product closed form.
  */
 #include <stdint.h>
 #include <stddef.h>

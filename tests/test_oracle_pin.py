@@ -152,6 +152,76 @@ def test_oracle_brute_force_python(oracle):
     assert np.array_equal(got, want)
 
 
+def test_oracle_three_contracted_indices_brute_force(oracle):
+    """The generic branch (three or more summed indices: an odometer with the FIRST listed index outermost): a loop nest
+    written out by hand with that order, distinct extents and the summed indices in different places of the two inputs,
+    bit-exact in both element types and for both operators.  A swapped pair of input strides or a reversed odometer
+    changes the summation order or the operands and fails the comparison."""
+    for op, dtype in (("+=", np.float64), ("-=", np.float64), ("+=", np.float32), ("-=", np.float32)):
+        text = "t3 [a,3,b,2] %s sum(e,4,d,2,f,3) * t2 [d,a,f,e] * v2 [f,e,b,d];" % op
+        expr = parse_expression(text)
+        a_, b_, e_, d_, f_ = sizes = [3, 2, 4, 2, 3]
+        C, A, B = inputs(expr, sizes, dtype)
+        want = C.copy()
+        for a, b in itertools.product(range(a_), range(b_)):
+            idx = a + a_ * b
+            for e in range(e_):                  # sum() order: e outermost, then d, then f
+                for d in range(d_):
+                    for f in range(f_):
+                        p = A[d + d_ * (a + a_ * (f + f_ * e))] * B[f + f_ * (e + e_ * (b + b_ * d))]
+                        want[idx] = want[idx] - p if op == "-=" else want[idx] + p
+        got = oracle.contract(expr, sizes, C.copy(), A, B)
+        assert got.dtype == dtype and np.array_equal(got, want), (op, dtype)
+        # the other summation order (f outermost) gives other bits for at least one element: the check above can tell them apart
+        other = C.copy()
+        for a, b in itertools.product(range(a_), range(b_)):
+            for f in range(f_):
+                for d in range(d_):
+                    for e in range(e_):
+                        p = A[d + d_ * (a + a_ * (f + f_ * e))] * B[f + f_ * (e + e_ * (b + b_ * d))]
+                        other[a + a_ * b] = other[a + a_ * b] - p if op == "-=" else other[a + a_ * b] + p
+        assert not np.array_equal(other, want)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_oracle_three_and_four_contracted_indices_vs_einsum_and_vs_the_two_index_loop(dtype, oracle):
+    """Generic branch against numpy einsum (values) and, with a unit extent added to the sum, against the two-index
+    branch that the reference's own loops pin (bits: the unit index adds no term and does not reorder the others)."""
+    text3 = "t3 [c,3,a,4,b,2] += sum(d,3,e,2,f,4) * t2 [e,a,d,f] * v2 [b,f,c,d,e];"
+    expr3 = parse_expression(text3)
+    sizes3 = [3, 4, 2, 3, 2, 4]
+    C, A, B = inputs(expr3, sizes3, dtype)
+    got = oracle.contract(expr3, sizes3, C.copy(), A, B)
+    assert helpers.rel_error(got, helpers.einsum_reference(expr3, sizes3, C, A, B)) < (1e-13 if dtype == np.float64 else 2e-6)
+    text4 = "t3 [a,2,b,3] -= sum(d,2,e,3,f,2,g,3) * t2 [g,a,e,d,f] * v2 [f,d,b,g,e];"
+    expr4 = parse_expression(text4)
+    sizes4 = [2, 3, 2, 3, 2, 3]
+    C, A, B = inputs(expr4, sizes4, dtype)
+    got = oracle.contract(expr4, sizes4, C.copy(), A, B)
+    assert helpers.rel_error(got, helpers.einsum_reference(expr4, sizes4, C, A, B)) < (1e-13 if dtype == np.float64 else 2e-6)
+    # sum(e, u, d) with extent(u) = 1 in either input  ==  sum(e, d), bit for bit
+    two = parse_expression("t3 [a,3,b,2,c,4] += sum(e,3,d,2) * t2 [a,d,e,c] * v2 [e,b,d];")
+    three = parse_expression("t3 [a,3,b,2,c,4] += sum(e,3,u,1,d,2) * t2 [a,u,d,e,c] * v2 [e,b,d,u];")
+    C, A, B = inputs(two, [3, 2, 4, 3, 2], dtype)
+    assert np.array_equal(oracle.contract(three, [3, 2, 4, 3, 1, 2], C.copy(), A, B), oracle.contract(two, [3, 2, 4, 3, 2], C.copy(), A, B))
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_oracle_without_contracted_index_is_the_outer_product(dtype, oracle):
+    """No summed index (the grammar cannot say it, the descriptor can): C[a,b,c] +/-= A[c,a] * B[b], one multiply and one
+    add per element, which numpy does with the same two roundings."""
+    for op in ("+=", "-="):
+        expr = {"out": "t3", "op": op, "a": "t2", "b": "v2", "out_idx": ["a", "b", "c"], "sum_idx": [],
+                "a_idx": ["c", "a"], "b_idx": ["b"], "all_idx": ["a", "b", "c"]}
+        sizes = [3, 4, 2]
+        C, A, B = inputs(expr, sizes, dtype)
+        got = oracle.contract(expr, sizes, C.copy(), A, B).reshape((3, 4, 2), order="F")
+        Af, Cf = A.reshape((2, 3), order="F"), C.reshape((3, 4, 2), order="F")
+        prod = (Af.T[:, None, :] * B[None, :, None]).astype(dtype)              # [a, b, c], rounded once
+        want = (Cf - prod if op == "-=" else Cf + prod).astype(dtype)
+        assert got.dtype == dtype and np.array_equal(got, want)
+
+
 def test_oracle_closed_forms(oracle):
     text = "t3 [a,4,b,3,c,5] += sum(d,7) * t2 [b,d,a] * v2 [d,c];"
     expr = parse_expression(text)
