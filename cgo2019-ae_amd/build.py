@@ -74,16 +74,76 @@ def tuned_map(entry):
     return hit["map"] if hit else None
 
 
+RESOURCE_FLAG = "-Rpass-analysis=kernel-resource-usage"
+
+
+def kernel_resources(remarks):
+    """hipcc's per-kernel resource remarks (the counterpart of the reference's `nvcc -Xptxas -v`,
+    cogent/Makefile:16) as {kernel: {"vgprs", "agprs", "scratch_bytes", "occupancy", "lds_bytes"}}; kernel names
+    are shortened to the template and its boolean arguments."""
+    import re
+    out, cur = {}, None
+    keys = {"VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch_bytes",
+            "Occupancy [waves/SIMD]": "occupancy", "LDS Size [bytes/block]": "lds_bytes", "VGPRs Spill": "vgpr_spills"}
+    for line in remarks.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", line)
+        if m:
+            sym = m.group(1)
+            base = re.search(r"(tc_\w+?_kernel|cogent_\w+_kernel)", sym)
+            flags = re.findall(r"Lb([01])", sym)
+            cur = (base.group(1) if base else sym) + ("<" + ",".join(flags) + ">" if flags else "")
+            if "IdE" in sym and not flags: cur += "<f64>"
+            if "IfE" in sym and not flags: cur += "<f32>"
+            out[cur] = {}
+            continue
+        m = re.search(r"remark:\s+([A-Za-z \[\]/]+): (\d+)", line)
+        if m and cur is not None and m.group(1).strip() in keys:
+            out[cur][keys[m.group(1).strip()]] = int(m.group(2))
+    return out
+
+
+def hot_kernel(info, sizes):
+    """The kernel instantiation the launcher picks for these extents (tc_launch.hpp: streaming kernel when the object
+    has one and the extents give full tiles and its K-block count; else the per-tile kernel's variant by divisibility)."""
+    m = info["mapping"]
+    ext = dict(zip(info["out_idx"] + info["sum_idx"], sizes))
+    div = lambda side: all(ext[n] % t == 0 for n, t in m[side])
+    nkb = 1
+    for n, t in m["k"]:
+        nkb *= -(-ext[n] // t)
+    swp = int(bool(m["swapped_roles"]) and ext[info["out_idx"][0]] % 4 == 0)
+    if m["stream"][0] > 0 and div("x") and div("y") and div("k") and nkb == m["stream"][0]:
+        return "tc_stream_kernel<%d>" % swp
+    bx, by, bk = m["block_tile"]
+    px, py, pk = m["padded"]
+    ext_full = int(div("x") and div("y") and bx == px and by == py)
+    int_full = int(div("k") and bk == pk)
+    return "tc_mfma_kernel<%d,%d,%d,%d>" % (ext_full, int_full, int(nkb == 1), swp)
+
+
 def emit_and_compile(entry):
+    """Emits and compiles one expression.  The compiler's resource report of every kernel in the object goes to
+    lib/<name>.resources.json ("hot" names the instantiation that runs at the entry's benchmark extents).  If THAT
+    kernel spills registers to scratch memory the build fails (such kernels ran 15 to 20 times slower when they were
+    measured) unless the entry says "allow_scratch"; spills in the variants for other extents are recorded only."""
     name = entry["name"]
     hip = os.path.join(GEN, name + ".hip")
     cmd = [os.path.join(BIN, "cogent_gen"), name, os.path.join(EXPR, entry["file"]),
-           str(entry.get("config", -1)), "-1", entry["dtype"], "-o", hip, "--name", name]
+           str(entry.get("config", -1)), "-1", entry["dtype"], "-o", hip, "--name", name, "--json"]
     spec = entry.get("map") or tuned_map(entry)
     if spec:
         cmd += ["--map", spec]
-    run(cmd)
-    run(["hipcc"] + HIPCC_FLAGS + ["-o", os.path.join(LIB, name + ".so"), hip])
+    plan = json.loads(run(cmd))
+    remarks = run(["hipcc"] + HIPCC_FLAGS + [RESOURCE_FLAG, "-o", os.path.join(LIB, name + ".so"), hip])
+    res = kernel_resources(remarks)
+    spilling = sorted(k for k, v in res.items() if v.get("scratch_bytes", 0) > 0 and k.startswith(("tc_mfma", "tc_stream", "tc_group")))
+    hot = hot_kernel(plan, entry["bench_sizes"]) if "mapping" in plan else None      # (a fused group has one kernel of its own)
+    with open(os.path.join(LIB, name + ".resources.json"), "w") as f:
+        json.dump({"hot": hot, "spilling": spilling, "kernels": res}, f, indent=1, sort_keys=True)
+    bad = [k for k in spilling if hot is None or k == hot]
+    if bad and not entry.get("allow_scratch"):
+        raise RuntimeError("%s: the kernel for its benchmark extents spills registers to scratch memory: %s (mapping %s)"
+                           % (name, ", ".join(bad), spec or "by the model"))
     return name
 
 

@@ -179,6 +179,16 @@ class Expression:
         self.info = json.loads(self.lib.cogent_info().decode())
         self.dtype = self.info["dtype"]
 
+    @property
+    def resources(self):
+        """hipcc's resource report of the object's kernels, written next to it by build.py: {"hot": the instantiation that
+        runs at the benchmark extents, "spilling": kernels with scratch use, "kernels": {name: {vgprs, scratch_bytes, ..}}}."""
+        path = self.path[:-3] + ".resources.json"
+        if not os.path.exists(path):
+            raise CogentError("no resource report next to %s (built by hand?)" % self.path)
+        with open(path) as f:
+            return json.load(f)
+
     def last_error(self):
         return self.lib.cogent_last_error().decode()
 

@@ -238,15 +238,22 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
         i, spec = args
         hip = os.path.join(out, "cand_%02d.hip" % i)
         so = os.path.join(out, "cand_%02d.so" % i)
-        r = subprocess.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", hip, "--name", name, "--map", spec],
-                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        r = subprocess.run([gen, name, src, "-1", "-1", entry["dtype"], "-o", hip, "--name", name, "--map", spec, "--json"],
+                           stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
         if r.returncode:
-            return {"i": i, "spec": spec, "error": "generator: " + r.stdout.strip()}
-        r = subprocess.run(["hipcc"] + b.HIPCC_FLAGS + ["-o", so, hip], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+            return {"i": i, "spec": spec, "error": "generator: " + (r.stderr + r.stdout).strip()}
+        plan = json.loads(r.stdout)
+        r = subprocess.run(["hipcc"] + b.HIPCC_FLAGS + [b.RESOURCE_FLAG, "-o", so, hip], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         os.remove(hip)
         if r.returncode:
             return {"i": i, "spec": spec, "error": "hipcc: " + r.stdout[-400:]}
-        return {"i": i, "spec": spec, "so": os.path.basename(so)}
+        # a candidate whose kernel for the benchmark extents spills registers is not worth the GPU's time
+        hot = b.hot_kernel(plan, entry["bench_sizes"])
+        res = b.kernel_resources(r.stdout).get(hot, {})
+        if res.get("scratch_bytes", 0) > 0:
+            os.remove(so)
+            return {"i": i, "spec": spec, "error": "%s spills %d bytes per lane to scratch memory" % (hot, res["scratch_bytes"])}
+        return {"i": i, "spec": spec, "so": os.path.basename(so), "vgprs": res.get("vgprs"), "occupancy": res.get("occupancy")}
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         index = list(ex.map(one, enumerate(specs)))

@@ -232,7 +232,7 @@ bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const 
     if (acc_regs > 256 || (m.from_spec ? acc_regs + 56 > reg_budget : acc_regs * 2 > reg_budget)) { err = "accumulator tiles exceed the register budget per lane"; return false; }
     if (m.layx < 0 || m.layx > 1 || m.layy < 0 || m.layy > 1) { err = "unknown LDS layout"; return false; }
     if (m.SK < 1 || m.SK > 64) { err = "split-K factor outside 1..64"; return false; }
-    if (m.MINW < 1 || m.MINW > 8 || m.MINW * ceil_div(m.WX * m.WY, arch.simd_per_cu) > 8) { err = "wavefronts per SIMD outside what a block of this size allows"; return false; }
+    if (m.MINW < 1 || m.MINW > 8) { err = "wavefronts per SIMD outside 1..8"; return false; }
     return true;
 }
 
@@ -587,6 +587,9 @@ static bool plan_stream(const Contraction& c, DType t, const ArchGfx950& arch, M
     const int waves = m.WX * m.WY;
     const int bpc = std::max(1, std::min((int)(arch.lds_bytes_per_cu / bytes), arch.max_waves_per_cu / 2 / waves));
     m.SMW = std::max(1, std::min(4, (bpc * waves + arch.simd_per_cu - 1) / arch.simd_per_cu));
+    // mw= asks for more resident wavefronts per SIMD (fewer registers each, more workgroups per CU): for the
+    // HBM-bound shapes with small accumulator tiles the memory system wants as many wavefronts in flight as fit
+    if (m.MINW > 1) m.SMW = std::min(8, m.MINW);
     return true;
 }
 

@@ -41,6 +41,22 @@ def test_every_expression_object_exports_the_entry_points():
             assert s in syms, (e["name"], s)
 
 
+def test_no_benchmark_kernel_spills_registers():
+    """build.py keeps hipcc's per-kernel resource report (the counterpart of the reference's `nvcc -Xptxas -v`,
+    cogent/Makefile:16) next to every object and fails on a spilling kernel; here: the report exists for every object, names
+    the instantiation its benchmark extents run, and that one uses no scratch memory and fits the register file."""
+    import cogent_mi355
+    for e in cogent_mi355.manifest():
+        res = cogent_mi355.Expression.resources.fget(type("P", (), {"path": os.path.join(PKG, "lib", e["name"] + ".so")})())
+        hot = res["hot"]
+        assert hot in res["kernels"], (e["name"], hot)
+        k = res["kernels"][hot]
+        assert k["scratch_bytes"] == 0 or e.get("allow_scratch"), (e["name"], hot, k)
+        assert 0 < k["vgprs"] + k.get("agprs", 0) <= 512 and k["occupancy"] >= 1
+        if e["name"].startswith("cfg"):
+            assert hot not in res["spilling"]
+
+
 def test_driver_library_exports():
     out = subprocess.run(["nm", "-D", "--defined-only", os.path.join(PKG, "lib", "libcogent_driver.so")],
                          stdout=subprocess.PIPE, text=True, check=True).stdout

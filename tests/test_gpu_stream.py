@@ -19,7 +19,7 @@ STREAMING = ["cfg2_f64", "var_cfg2_stream96_f64", "var_cfg4_stream_f32", "var_st
              "var_tccg09_stream_pad_f64",    # the X panel resident, its 72 columns padded to 80
              "var_cfg4_stream_pad_f32",      # fp32, 128-bit C accesses, a Y tile of 24 rows padded to 32
              "var_cfg2_stream_cd2_f64",      # C read two tiles ahead (runs of 12 and 9 tiles: both parities end a run)
-             "var_tccg11_stream_y_ov_f64"]   # Y panel loaded behind the first tile, interleaved runs, C two tiles ahead
+             "var_tccg11_stream_y_ov_f64"]   # Y panel loaded behind the first tile, interleaved runs
 
 
 def _check(name, sizes, tools, oracle, variant=None, expect=None):
