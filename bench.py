@@ -33,7 +33,7 @@ HEADLINE = "cfg2_f64"
 def read_traffic(name):
     """HBM bytes per launch from the rocprofv3 counter summary under profiles/ (FETCH_SIZE and WRITE_SIZE of the
     contraction kernel, each scaled by what the same counter reads for a plain copy of known size), or None."""
-    path = os.path.join(ROOT, "profiles", "traffic_%s.txt" % name)
+    path = os.path.join(ROOT, "profiles", "counters_%s.txt" % name)
     if not os.path.exists(path):
         return None
     for line in open(path):
@@ -44,7 +44,7 @@ def read_traffic(name):
 
 def read_mfma_busy(name):
     """Fraction of the kernel's active cycles with the matrix cores busy, from the counter summary under profiles/, or None."""
-    path = os.path.join(ROOT, "profiles", "mfma_%s.txt" % name)
+    path = os.path.join(ROOT, "profiles", "counters_%s.txt" % name)
     if not os.path.exists(path):
         return None
     for line in open(path):
