@@ -196,7 +196,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
     ap.add_argument("--workload", default=HEADLINE, help="expression object to use as the headline workload")
     ap.add_argument("--suite", default="", help="'fused': time the fused groups of the manifest; 'tccg': time the 48 TCCG contractions at the sizes of the reference's "
-                    "bench script (cogent/bench_tccg.sh:5-54) and print one JSON line with the table, instead of the headline run")
+                    "bench script (cogent/bench_tccg.sh:5-54) and print one JSON line with the table, instead of the headline run; "
+                    "any other value: the manifest entries whose names start with it (comma-separated prefixes, e.g. 'smallk,ext4')")
     ap.add_argument("--ceilings", action="store_true",
                     help="only run the memory yardsticks: plain copy and bare read-modify-write streams (flat, and in the streaming "
                          "kernel's tiles of config 2's output) at the output sizes of the HBM-bound configs; one JSON line")
@@ -290,7 +291,7 @@ def main():
     if args.suite:
         rows = []
         for e in pkg.manifest():
-            if not e["name"].startswith(args.suite):
+            if not e["name"].startswith(tuple(args.suite.split(","))):
                 continue
             wl = Workload(pkg, tools, e, e["bench_sizes"])
             r = time_workload(driver, wl, max(1, min(args.warmup, 3)), max(3, min(args.steps, 20)))

@@ -165,7 +165,8 @@ def build_all(jobs=8, only=None):
         sys.path.insert(0, HERE)
         from cogent_mi355 import tuner
         for name, k in TUNING_SETS.items():
-            bad = [c for c in tuner.prepare(name, k, jobs=jobs) if "so" not in c]
+            # (a candidate whose kernel spills registers is dropped by the tuner on purpose: not a build failure)
+            bad = [c for c in tuner.prepare(name, k, jobs=jobs) if "so" not in c and "spills" not in c.get("error", "")]
             if bad:
                 raise RuntimeError("tuning candidate failed to build: %r" % bad[0])
     return [e["name"] for e in entries]

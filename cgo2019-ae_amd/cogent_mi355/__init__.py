@@ -193,9 +193,9 @@ class Expression:
         return self.lib.cogent_last_error().decode()
 
     def last_kernel(self):
-        """Kernel launched by this thread's last call: 'none', 'plain', 'tiled' or 'stream'."""
+        """Kernel launched by this thread's last call: 'none', 'plain', 'tiled', 'stream' or 'valu'."""
         self.lib.cogent_last_kernel.restype = ctypes.c_int
-        return ("none", "plain", "tiled", "stream")[self.lib.cogent_last_kernel()]
+        return ("none", "plain", "tiled", "stream", "valu")[self.lib.cogent_last_kernel()]
 
     def entry(self, sizes, c_ptr, a_ptr, b_ptr):
         """sd_t_d2_fusion_(size..., C, A, B, 1, -1) on device addresses; returns the status code."""

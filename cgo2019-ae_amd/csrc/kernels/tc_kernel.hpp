@@ -814,4 +814,81 @@ void tc_plain_kernel(T* __restrict__ C, const T* __restrict__ A, const T* __rest
     C[lin] = acc;
 }
 
+// ---------------------------------------------------------------------------
+// VALU streaming kernel, written for contracted ranges too short to fill one step of a matrix instruction (fewer than
+// 4 terms per output element: the fp64 and fp32 MFMAs are 4 deep).  Such a contraction is a read-modify-write stream of
+// C with two or three multiply-adds per element attached.  Measured, the tiled kernel with its slices zero-padded to
+// one matrix step is still the faster one there (see tc_launch.hpp), so this kernel runs only on request
+// (variant 3): as a second bit-exact check kernel, 2 to 5 times faster than the plain one.  Every lane owns V
+// consecutive elements of C's fastest index (one 16-byte access), U such vectors in flight, blocks walk C in its
+// memory order like a plain copy kernel, and the few input elements an output element needs are read straight
+// through L1/L2 (the inputs of such a shape are tiny next to C).  The terms are added in sum() order with separately
+// rounded multiply and add, which is the reference host loop's arithmetic
+// (cogent/drivers/tccg/code_main_tccg_01.c:117-133): the result is bit-exact with the oracle.  No cross-lane
+// reduction is needed, the whole contracted range sits in one lane.
+// The reference's register-tile FMA loop is the counterpart: cogent/src/codes/kernels/tc_code_kernel_compute.py:4-204.
+struct TcValuDims {
+    int n_out, n_int;
+    int ext_out[TC_MAXI], sA_out[TC_MAXI], sB_out[TC_MAXI];     // C's indices in memory order: extent, stride in A, in B
+    int ext_k[TC_MAXI], sA_k[TC_MAXI], sB_k[TC_MAXI];           // contracted indices in sum() order
+    int sign;
+    unsigned plane;        // elements of C's three fastest indices together: what a lane decodes for itself
+    unsigned chunks;       // blocks per plane
+    unsigned nplanes;      // product of the remaining output extents
+    int ktotal;
+};
+
+template <class T, int V, int U>
+__global__ __launch_bounds__(256)
+void tc_valu_kernel(T* __restrict__ C, const T* __restrict__ A, const T* __restrict__ B, const TcValuDims p)
+{
+    typedef T TV __attribute__((ext_vector_type(V), aligned(sizeof(T) * V)));
+    const unsigned pl = blockIdx.x / p.chunks, ch = blockIdx.x % p.chunks;
+    // the block's plane: indices 3.. are the same for all its lanes
+    long long baseA = 0, baseB = 0;
+    {
+        unsigned r = pl;
+        for (int i = 3; i < p.n_out; i++) {
+            const unsigned e = (unsigned)p.ext_out[i], q = r % e;
+            r /= e;
+            baseA += (long long)q * p.sA_out[i];
+            baseB += (long long)q * p.sB_out[i];
+        }
+    }
+    T* const Cp = C + (long long)pl * p.plane;
+    const T* const Ap = A + uniform64(baseA);
+    const T* const Bp = B + uniform64(baseB);
+    const unsigned e0 = (unsigned)p.ext_out[0], e1 = p.n_out > 1 ? (unsigned)p.ext_out[1] : 1u;
+    const int sA0 = p.sA_out[0], sB0 = p.sB_out[0];
+    const int sA1 = p.n_out > 1 ? p.sA_out[1] : 0, sB1 = p.n_out > 1 ? p.sB_out[1] : 0;
+    const int sA2 = p.n_out > 2 ? p.sA_out[2] : 0, sB2 = p.n_out > 2 ? p.sB_out[2] : 0;
+    TV c[U];
+    unsigned pos[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        pos[u] = ((ch * U + u) * 256u + threadIdx.x) * V;
+        if (pos[u] < p.plane) c[u] = __builtin_nontemporal_load((const TV*)(Cp + pos[u]));
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if (pos[u] >= p.plane) continue;
+        const unsigned i0 = pos[u] % e0, t = pos[u] / e0, i1 = t % e1, i2 = t / e1;
+        const int oa = (int)i0 * sA0 + (int)i1 * sA1 + (int)i2 * sA2;
+        const int ob = (int)i0 * sB0 + (int)i1 * sB1 + (int)i2 * sB2;
+        int k[TC_MAXI];
+        for (int i = 0; i < p.n_int; i++) k[i] = 0;
+        for (int kk = 0; kk < p.ktotal; kk++) {
+            int ka = oa, kb = ob;
+            for (int i = 0; i < p.n_int; i++) { ka += k[i] * p.sA_k[i]; kb += k[i] * p.sB_k[i]; }
+#pragma unroll
+            for (int v = 0; v < V; v++) {
+                const T prod = tc_mul_rn(Ap[ka + v * sA0], Bp[kb + v * sB0]);
+                c[u][v] = tc_add_rn(c[u][v], p.sign < 0 ? -prod : prod);
+            }
+            for (int j = p.n_int - 1; j >= 0; j--) { if (++k[j] < p.ext_k[j]) break; k[j] = 0; }
+        }
+        __builtin_nontemporal_store(c[u], (TV*)(Cp + pos[u]));
+    }
+}
+
 }  // namespace cogent

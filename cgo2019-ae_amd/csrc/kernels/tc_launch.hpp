@@ -44,10 +44,14 @@ inline int tc_check_launch(const char* what)
     return TC_ERR_LAUNCH;
 }
 
-enum TcVariant { TC_VARIANT_AUTO = 0, TC_VARIANT_PLAIN = 1, TC_VARIANT_TILED = 2 };
+enum TcVariant { TC_VARIANT_AUTO = 0, TC_VARIANT_PLAIN = 1, TC_VARIANT_TILED = 2, TC_VARIANT_VALU = 3 };
+// The VALU streaming kernel is never taken by TC_VARIANT_AUTO: measured at contracted extents 1, 2 and 3 (which do not
+// fill the 4-deep step of the fp64 / fp32 matrix instructions) it is 18 to 56 % SLOWER than the tiled kernel with the
+// slices zero-padded to one step (72^4 outer product 131 vs 111 us, 16^6 fp64 with 2 terms 70 vs 51 us, 16^6 fp32 with
+// 3 terms 51 vs 33 us): its per-element gathers of the inputs cost more issue slots than a padded matrix step.
 
 // Which kernel the last call of this thread launched (0: none yet, or the call returned before a launch).
-enum TcKernelKind { TC_KERNEL_NONE = 0, TC_KERNEL_PLAIN = 1, TC_KERNEL_TILED = 2, TC_KERNEL_STREAM = 3 };
+enum TcKernelKind { TC_KERNEL_NONE = 0, TC_KERNEL_PLAIN = 1, TC_KERNEL_TILED = 2, TC_KERNEL_STREAM = 3, TC_KERNEL_VALU = 4 };
 inline int& tc_last_kernel() { static thread_local int kind = TC_KERNEL_NONE; return kind; }
 
 template <class Cfg, bool ONE_KB, bool SWP>
@@ -167,7 +171,7 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     typedef typename Cfg::T T;
     tc_error_buffer()[0] = 0;
     tc_last_kernel() = TC_KERNEL_NONE;
-    if (variant < 0 || variant > 2) return tc_fail(TC_ERR_BAD_VARIANT, "unknown kernel variant");
+    if (variant < 0 || variant > 3) return tc_fail(TC_ERR_BAD_VARIANT, "unknown kernel variant");
     for (int i = 0; i < Cfg::NIDX; i++)
         if (sizes[i] < 0) return tc_fail(TC_ERR_NEGATIVE_EXTENT, "negative extent");
     // empty output or empty sum: C is left as it is
@@ -208,6 +212,41 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
                            (T*)C, (const T*)A, (const T*)B, p);
         tc_last_kernel() = TC_KERNEL_PLAIN;
         return tc_check_launch("plain kernel launch failed");
+    }
+
+    // Asked for: the VALU streaming kernel.  Blocks of 256 lanes walk C in memory order, 16 bytes per lane and 8 such
+    // vectors in flight; a lane decodes the three fastest output indices itself.
+    {
+        int64_t kterms = 1;
+        for (int j = 0; j < Cfg::NK; j++) kterms *= sizes[Cfg::sum_id(j)];
+        if (variant == TC_VARIANT_VALU) {
+            if (kterms > lim) return tc_fail(TC_ERR_TOO_LARGE, "contracted range too large");
+            TcValuDims p;
+            memset(&p, 0, sizeof(p));
+            p.n_out = Cfg::CR; p.n_int = Cfg::NK; p.sign = Cfg::SIGN; p.ktotal = (int)kterms;
+            int64_t plane = 1, nplanes = 1;
+            for (int j = 0; j < Cfg::CR; j++) {
+                const int id = Cfg::c_id(j);
+                p.ext_out[j] = sizes[id]; p.sA_out[j] = (int)sA[id]; p.sB_out[j] = (int)sB[id];
+                if (j < 3) plane *= sizes[id]; else nplanes *= sizes[id];
+            }
+            for (int j = 0; j < Cfg::NK; j++) {
+                const int id = Cfg::sum_id(j);
+                p.ext_k[j] = sizes[id]; p.sA_k[j] = (int)sA[id]; p.sB_k[j] = (int)sB[id];
+            }
+            constexpr int VFULL = 16 / (int)sizeof(T), U = 8;
+            const bool vec = (sizes[Cfg::c_id(0)] % VFULL == 0) && (((uintptr_t)C & 15) == 0);
+            const int64_t per_block = 256 * (int64_t)(vec ? VFULL : 1) * U;
+            const int64_t chunks = (plane + per_block - 1) / per_block;
+            if (chunks * nplanes > lim) return tc_fail(TC_ERR_TOO_LARGE, "grid too large");
+            p.plane = (unsigned)plane; p.chunks = (unsigned)chunks; p.nplanes = (unsigned)nplanes;
+            tc_clear_hip_error();
+            const dim3 g((unsigned)(chunks * nplanes)), b(256);
+            if (vec) hipLaunchKernelGGL((tc_valu_kernel<T, VFULL, U>), g, b, 0, stream, (T*)C, (const T*)A, (const T*)B, p);
+            else     hipLaunchKernelGGL((tc_valu_kernel<T, 1, U>), g, b, 0, stream, (T*)C, (const T*)A, (const T*)B, p);
+            tc_last_kernel() = TC_KERNEL_VALU;
+            return tc_check_launch("VALU kernel launch failed");
+        }
     }
 
     TcDims d;

@@ -125,7 +125,11 @@ void cogent_fill_uniform_f32(float* dst, long long n, unsigned long long seed);
  * panel-resident streaming kernel when it was emitted and the extents give full
  * tiles and its K-block count, otherwise the tiled MFMA kernel), 1 = plain
  * one-lane-per-element kernel whose summation order is the reference host
- * loop's, 2 = the tiled MFMA kernel with one workgroup per output tile.
+ * loop's, 2 = the tiled MFMA kernel with one workgroup per output tile, 3 = the
+ * VALU streaming kernel (blocks walk C in memory order, every lane adds the terms of
+ * its own elements in sum() order with separately rounded multiply and add: bit-exact
+ * with the reference host loop; never taken by variant 0: even at contracted extents
+ * below the 4-deep step of the matrix instructions the tiled kernel measured faster).
  * Status codes: 0 ok, 1 null pointer / bad sizes[], 2 negative extent,
  * 3 tensor or grid too large (2^31 elements, or a tile of the mapping spanning 4 GB or more
  * of a tensor), 4 launch failed, 5 bad variant. */
@@ -147,7 +151,8 @@ int cogent_run_noalloc(const int* sizes, int n_sizes, void* C, const void* A, co
 int cogent_num_indices(void);
 const char* cogent_last_error(void);   /* message of the last failing call on this thread */
 int cogent_last_kernel(void);          /* kernel launched by this thread's last call: 0 none, 1 plain, 2 tiled (one
-                                          workgroup per output tile), 3 panel-resident streaming kernel */
+                                          workgroup per output tile), 3 panel-resident streaming kernel,
+                                          4 VALU streaming kernel */
 const char* cogent_expression(void);   /* the expression this object was emitted for      */
 const char* cogent_info(void);         /* JSON: the mapping compiled into this object     */
 

@@ -28,7 +28,7 @@ def test_status_codes(tools):
     assert ex.entry([4, 5, 6, 7], None, dA.ptr, dB.ptr) == 1 and "null" in ex.last_error()
     assert ex.entry([4, 5, 6, 7], dC.ptr, None, dB.ptr) == 1
     assert ex.entry([4, -5, 6, 7], dC.ptr, dA.ptr, dB.ptr) == 2 and "negative" in ex.last_error()
-    assert ex.run([4, 5, 6, 7], dC.ptr, dA.ptr, dB.ptr, None, 9) == 5
+    assert ex.run([4, 5, 6, 7], dC.ptr, dA.ptr, dB.ptr, None, 9) == 5 and ex.run([4, 5, 6, 7], dC.ptr, dA.ptr, dB.ptr, None, -1) == 5
     assert ex.run([4, 5, 6], dC.ptr, dA.ptr, dB.ptr, None, 0) == 1          # wrong number of extents
     # 2^31 elements or more in a tensor: refused before anything is launched
     assert ex.entry([2048, 2048, 1024, 2], dC.ptr, dA.ptr, dB.ptr) == 3 and "2^31" in ex.last_error()

@@ -18,7 +18,7 @@ def configs():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     with open(os.path.join(root, "cgo2019-ae_amd", "expressions", "manifest.json")) as f:
         return [(e["name"], e["bench_sizes"], e.get("c_init") == "seeded") for e in json.load(f)["expressions"]
-                if e["name"].startswith("cfg")]
+                if e["name"].startswith(("cfg", "smallk", "ext4"))]
 
 
 @pytest.mark.parametrize("name,sizes,seeded", configs(), ids=[c[0] for c in configs()])
@@ -92,3 +92,26 @@ def test_full_size_closed_form_and_linearity(name, tools):
     else:
         assert bool((c2 == 2 * c1).all())
     assert float(c1.abs().max()) > 0
+
+
+@pytest.mark.parametrize("name", ["cfg5_1_f64", "cfg4_16_f32", "cfg2_f64", "smallk2_f64"])
+@pytest.mark.parametrize("k", [1, 2, 3, 5, 7])
+def test_contracted_extents_that_do_not_fill_a_matrix_step(name, k, tools, oracle):
+    """Contracted extents below the 4-deep step of the fp64 / fp32 matrix instructions, and odd ones above it: the
+    slices are zero-padded to the step in LDS (no separate small-K kernel: a padded step costs nothing next to the
+    output traffic, see the measured small-K rows of the benchmark).  Every element against the oracle."""
+    import cogent_mi355 as pkg
+    from gpu_common import make_inputs, run_entry
+    ex = pkg.Expression(name)
+    expr = helpers.parse_expression(pkg.expression_text(name))
+    tiles = {n: t for side in ("x", "y", "k") for n, t in ex.info[side]}
+    sizes = [k if n in expr["sum_idx"] else min(2 * tiles[n], 24) for n in expr["all_idx"]]
+    dtype = np.float64 if ex.dtype == "f64" else np.float32
+    print("[gpu] small contracted extent %s sizes=%s" % (name, sizes), flush=True)
+    C, A, B = make_inputs(tools, expr, sizes, dtype)
+    got = run_entry(ex, sizes, C, A, B)
+    want = oracle.contract(expr, sizes, C.copy(), A, B)
+    assert helpers.rel_error(got, want) <= TOL[ex.dtype]
+    if k == 1:
+        # a single term per element: one product and one sum, the oracle's two roundings or the fused one
+        assert helpers.rel_error(got, want) <= (3e-16 if ex.dtype == "f64" else 2e-7)

@@ -72,6 +72,17 @@ def test_plain_kernel_is_bit_exact(name, tools, oracle):
 
 
 @pytest.mark.parametrize("name", all_names())
+def test_valu_streaming_kernel_is_bit_exact(name, tools, oracle):
+    """variant 3: blocks walk C in memory order, every lane sums its elements' terms in sum() order with separately
+    rounded multiply and add.  Ragged sizes (scalar accesses) and sizes whose fastest extent allows 16-byte accesses."""
+    pkg = _pkg()
+    n = pkg.Expression(name).n
+    ex = check(name, SMALL[:n], tools, oracle, variant=3, exact=True)
+    assert ex.last_kernel() == "valu"
+    check(name, ([8] + SMALL[1:])[:n], tools, oracle, variant=3, exact=True)
+
+
+@pytest.mark.parametrize("name", all_names())
 def test_exact_tile_multiples(name, tools, oracle):
     """Extents equal to the compiled tiles (twice the tile on the first and the last index when small)."""
     pkg = _pkg()

@@ -64,7 +64,9 @@ def test_prepared_set_of_the_build_is_complete():
         idx = json.load(open(os.path.join(d, "index.json")))
         assert idx["name"] == name and len(idx["candidates"]) >= k
         for c in idx["candidates"]:
-            assert "error" not in c and os.path.exists(os.path.join(d, c["so"]))
+            # a candidate is built, or was dropped because the kernel for the benchmark extents spills registers
+            assert ("error" in c and "spills" in c["error"]) or os.path.exists(os.path.join(d, c["so"])), c
+        assert sum(1 for c in idx["candidates"] if "so" in c) >= k
         assert len({c["spec"] for c in idx["candidates"]}) == len(idx["candidates"])
 
 
@@ -89,6 +91,9 @@ def test_measure_times_verified_candidates_and_records_the_fastest(tmp_path):
     print("[gpu] tuner.measure cfg5_1_f64", flush=True)
     rep = tuner.measure("cfg5_1_f64", warmup=2, iters=10, cache_path=cache)
     rows = rep["candidates"]
+    dropped = [r for r in rows if "so" not in r]
+    assert all("spills" in r["error"] for r in dropped), dropped               # the only reason a candidate may be missing
+    rows = [r for r in rows if "so" in r]
     assert len(rows) >= 3 and all(r["ok"] for r in rows), rows
     assert all(r["max_rel_err"] <= 1e-12 for r in rows)
     best = min(rows, key=lambda r: r["mean_us"])
