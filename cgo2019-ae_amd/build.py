@@ -58,6 +58,12 @@ def build_host_tools():
          "-o", os.path.join(LIB, "libcogent_mi355.so")] + srcs)
     run(["g++", "-O2", "-std=c++17", "-Wall", "-o", os.path.join(BIN, "cogent_gen"),
          os.path.join(CSRC, "tc_cli.cpp"), "-L" + LIB, "-lcogent_mi355", "-Wl,-rpath,$ORIGIN/../lib"])
+    # the same generator with AddressSanitizer and UndefinedBehaviorSanitizer (host code only; the runtimes linked
+    # statically so that nothing has to be preloaded): parser, spec reader and emitter take untrusted text, and the
+    # CPU tests push the corpus and malformed input through this binary
+    run(["g++", "-O1", "-g", "-std=c++17", "-fopenmp", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+         "-fno-omit-frame-pointer", "-static-libasan", "-static-libubsan", "-o", os.path.join(BIN, "cogent_gen_san"),
+         os.path.join(CSRC, "tc_cli.cpp")] + srcs)
 
 
 # manifest entries whose top candidates are compiled ahead of time so that the tuner's measuring step

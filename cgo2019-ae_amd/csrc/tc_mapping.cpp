@@ -656,6 +656,17 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
     }
     if (m.MI < 0 || m.MI > 2) { err = "mapping spec: unknown matrix instruction"; return false; }
     if (m.x_ids.empty()) { err = "mapping spec must give x"; return false; }
+    // ranges first: everything below multiplies these numbers
+    {
+        long long vol = 1;
+        for (const std::vector<int>* tl : {&m.x_tiles, &m.y_tiles, &m.k_tiles})
+            for (int v : *tl) {
+                if (v < 1 || v > 65536) { err = "mapping spec: a tile outside 1..65536"; return false; }
+                vol *= v;
+                if (vol > (1LL << 24)) { err = "mapping spec: tile volume too large"; return false; }
+            }
+        if (m.WX < 1 || m.WY < 1 || m.TX < 1 || m.TY < 1 || m.WX > 16 || m.WY > 16 || m.TX > 64 || m.TY > 64) { err = "mapping spec: wavefront grid or MFMA tile count out of range"; return false; }
+    }
     const std::vector<int> xop = operand_order(c, m, true), yop = operand_order(c, m, false);
     m.layx = lx >= 0 ? lx : ((!m.k_ids.empty() && m.k_ids[0] == fvi(xop) && m.k_tiles[0] >= 4) ? 1 : 0);
     m.layy = ly >= 0 ? ly : ((!m.k_ids.empty() && m.k_ids[0] == fvi(yop) && m.k_tiles[0] >= 4) ? 1 : 0);

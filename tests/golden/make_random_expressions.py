@@ -6,7 +6,8 @@ import json
 import os
 import random
 
-HERE = os.path.dirname(os.path.abspath(__file__))
+# the files are written into the package's expression corpus
+HERE = os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))), "cgo2019-ae_amd", "expressions")
 LETTERS = "abcdefghijkl"
 
 
@@ -54,7 +55,7 @@ def main(n=12, seed=20190216):
         name = "rand_%02d_%s" % (k, "f64" if dtype == "DOUBLE" else "f32")
         fn = "rand_%02d.in" % k
         with open(os.path.join(HERE, fn), "w") as f:
-            f.write("# seeded random contraction %d (make_random.py, seed %d)\n%s\n" % (k, seed, text))
+            f.write("# seeded random contraction %d (tests/golden/make_random_expressions.py, seed %d)\n%s\n" % (k, seed, text))
         entries.append({"name": name, "file": fn, "dtype": dtype, "bench_sizes": sizes, "config_id": "random %d" % k})
     path = os.path.join(HERE, "manifest.json")
     m = json.load(open(path))

@@ -120,7 +120,7 @@ def test_odd_extents_mixed_full_and_partial(name, tools, oracle):
 
 @pytest.mark.parametrize("name", [n for n in all_names() if n.startswith("rand_")])
 def test_random_expressions_at_their_own_and_at_odd_sizes(name, tools, oracle):
-    """The seeded random expressions (expressions/make_random.py): at the sizes they were mapped for, and
+    """The seeded random expressions (written by tests/golden/make_random_expressions.py): at the sizes they were mapped for, and
     at odd sizes that divide none of their tiles."""
     pkg = _pkg()
     n = pkg.Expression(name).n
