@@ -61,19 +61,20 @@ template <class Term, int NARGS>
 __device__ __forceinline__ void term_setup(TermGeom<Term>& g, const TcGroupArgs<NARGS>& ga, const TcTermArgs& ta, const int* origin)
 {
     typedef typename Term::T T;
-    int64_t baseX = 0, baseY = 0;
+    // element offsets of the slices' origins: the host refuses inputs of 2^31 elements or more, so 32 bits hold them
+    unsigned baseX = 0, baseY = 0;
 #pragma unroll
     for (int i = 0; i < Term::NIDX; i++) {
         g.d.ext[i] = ga.ext[i]; g.d.nblk[i] = ga.nblk[i]; g.d.sC[i] = ga.sC[i]; g.d.sX[i] = ta.sX[i]; g.d.sY[i] = ta.sY[i];
         g.rem[i] = ga.ext[i] - origin[i];                     // contracted ids: origin 0
-        baseX += (int64_t)origin[i] * ta.sX[i];
-        baseY += (int64_t)origin[i] * ta.sY[i];
+        baseX += (unsigned)origin[i] * (unsigned)ta.sX[i];
+        baseY += (unsigned)origin[i] * (unsigned)ta.sY[i];
     }
     g.nkb = 1;
 #pragma unroll
     for (int i = 0; i < Term::NK; i++) g.nkb *= (ga.ext[Term::k_id(i)] + Term::k_tile(i) - 1) / Term::k_tile(i);
-    g.Xb = (const T*)ta.x + uniform64(baseX);
-    g.Yb = (const T*)ta.y + uniform64(baseY);
+    g.Xb = (const T*)ta.x + (size_t)(unsigned)__builtin_amdgcn_readfirstlane(baseX);
+    g.Yb = (const T*)ta.y + (size_t)(unsigned)__builtin_amdgcn_readfirstlane(baseY);
 }
 
 // One term: contract its slices for the block's C tile and add the result into the LDS copy of the tile.
@@ -182,8 +183,8 @@ void tc_group_kernel(typename G::T* __restrict__ C, const TcGroupArgs<(int)sizeo
 {
     typedef typename G::T T;
     constexpr int NT = G::NT, VOL = G::TILE_VOL;
-    __shared__ __attribute__((aligned(16))) T lds_c[VOL];
-    __shared__ __attribute__((aligned(16))) T lds_ops[G::LDS_OPS];
+    T* const lds_c = (T*)tc_dynamic_lds;                     // the copy of the C tile, then one operand region
+    T* const lds_ops = lds_c + VOL;
     const int tid = threadIdx.x;
 
     // which C tile: C's indices in C order, fastest first; XCD-contiguous ranges as in the single kernel
@@ -248,6 +249,242 @@ void tc_group_kernel(typename G::T* __restrict__ C, const TcGroupArgs<(int)sizeo
         const unsigned q = (unsigned)(tid + i * NT);
         unsigned off;
         if ((VOL % NT == 0 || q < (unsigned)VOL) && c_element(q, off)) Cb[off] = lds_c[q];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Pipelined form of the group kernel, for the common call: every term enabled and every term's contracted range in
+// one K block.  The serial form above pays, per term, an exposed gather of the two slices (an L2 round trip that
+// nothing overlaps) and three barriers for a fraction of a microsecond of matrix work.  Here the slices of term
+// t + 1 are requested BEFORE term t is contracted and go to a second operand region of the LDS after it, so that
+// a term costs one barrier and its gather hides behind the previous term's matrix instructions:
+//
+//     load(0); load(1); store(0 -> region 0); barrier
+//     for t: load(t + 2) | contract(t, region t % 2) | add into the LDS copy of C | store(t + 1 -> region (t + 1) % 2) | barrier
+//
+// (two register sets alternate, so a gather has two terms' time to arrive before its slices are needed in LDS)
+// The one barrier per term orders three things at once: region (t + 1) % 2 is complete before term t + 1 reads it,
+// term t's additions to the copy of C are visible before term t + 1 adds to other lanes' elements, and region
+// t % 2 has been read by everybody before term t + 2's slices overwrite it.
+// Registers per lane for a term's two slices in the pipelined kernel.  FULL: every tile of the call is whole (no
+// predicates), which also lets a lane fetch Operand::VW consecutive elements of the input's fastest index at once.
+// *p += v in LDS.  fp64: ONE instruction (the LDS unit adds; no value comes back) instead of read, add, write
+// (5 to 15 % faster for the group of nine fp64 terms, measured side by side on several tiles).  fp32: read, add, write -- the single-instruction form
+// measured 2.2 times SLOWER there (787 against 351 us for the nine fp32 terms, whatever the tile).  Every element of
+// the tile is added to by exactly one lane per term and barriers separate the terms, so the sum is deterministic.
+__device__ __forceinline__ void lds_accumulate(double* p, double v)
+{
+    (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void lds_accumulate(float* p, float v) { *p += v; }
+
+template <class Term, bool FULL> struct PipeSlots {
+    static constexpr int VX = slice_vw<Operand<Term, 0>, FULL, FULL>(), VY = slice_vw<Operand<Term, 1>, FULL, FULL>();
+    static constexpr int X = slice_slots<Term, Operand<Term, 0>, VX>(), Y = slice_slots<Term, Operand<Term, 1>, VY>();
+};
+
+template <class Term, bool FULL, int MAXX, int MAXY, int NARGS>
+__device__ __forceinline__ void group_load(typename Term::T (&px)[MAXX], typename Term::T (&py)[MAXY], const TcGroupArgs<NARGS>& ga,
+                                           const TcTermArgs& ta, const int* origin, int tid)
+{
+    TermGeom<Term> g;
+    term_setup<Term>(g, ga, ta, origin);
+    typedef PipeSlots<Term, FULL> S;
+    typename Term::T rx[S::X], ry[S::Y];
+    slice_load<Term, Operand<Term, 0>, FULL, FULL>(rx, g.Xb, g.d, g.rem, tid);
+    slice_load<Term, Operand<Term, 1>, FULL, FULL>(ry, g.Yb, g.d, g.rem, tid);
+#pragma unroll
+    for (int i = 0; i < S::X; i++) px[i] = rx[i];
+#pragma unroll
+    for (int i = 0; i < S::Y; i++) py[i] = ry[i];
+}
+
+template <class G, class Term, bool FULL, int MAXX, int MAXY, int NARGS>
+__device__ __forceinline__ void group_store(const typename Term::T (&px)[MAXX], const typename Term::T (&py)[MAXY], typename G::T* region,
+                                            const TcGroupArgs<NARGS>& ga, const TcTermArgs& ta, const int* origin, int tid)
+{
+    typedef typename G::T T;
+    typedef Operand<Term, 0> OX;
+    typedef Operand<Term, 1> OY;
+    constexpr int LDS_X = lds_elems<OX, Term::BKP>(), LDS_Y = lds_elems<OY, Term::BKP>();
+    constexpr bool PADDED = (Term::BKP != Term::BK) || (Term::BXP != Term::BX) || (Term::BYP != Term::BY);
+    static_assert(LDS_X + LDS_Y <= G::LDS_OPS, "operand slices exceed the group's LDS share");
+    TermGeom<Term> g;
+    term_setup<Term>(g, ga, ta, origin);
+    // the staging never writes the padding rows and columns: clear them (disjoint from what the staging writes)
+    if (PADDED) {
+        constexpr bool PX = (Term::BKP != Term::BK) || (Term::BXP != Term::BX), PY = (Term::BKP != Term::BK) || (Term::BYP != Term::BY);
+        if (PX) for (int i = tid; i < LDS_X; i += Term::NT) region[i] = (T)0;
+        if (PY) for (int i = tid; i < LDS_Y; i += Term::NT) region[LDS_X + i] = (T)0;
+        if (PX || PY) __syncthreads();
+    }
+    typedef PipeSlots<Term, FULL> S;
+    typename Term::T rx[S::X], ry[S::Y];
+#pragma unroll
+    for (int i = 0; i < S::X; i++) rx[i] = px[i];
+#pragma unroll
+    for (int i = 0; i < S::Y; i++) ry[i] = py[i];
+    slice_store<Term, OX, false, S::VX>(rx, region, g.d, tid);
+    slice_store<Term, OY, (Term::SIGN < 0), S::VY>(ry, region + LDS_X, g.d, tid);
+}
+
+template <class G, class Term, bool FULL, int NARGS>
+__device__ __forceinline__ void group_contract(typename G::T* lds_c, const typename G::T* region, const TcGroupArgs<NARGS>& ga,
+                                               const TcTermArgs& ta, const int* origin, int tid)
+{
+    typedef typename G::T T;
+    typedef Mfma<Term::MI> MM;
+    typedef typename MM::Acc Acc;
+    typedef Operand<Term, 0> OX;
+    typedef Operand<Term, 1> OY;
+    constexpr int MT = MM::MT, NREG = MM::NREG, KSTEP = MM::KSTEP, TX = Term::TX, TY = Term::TY;
+    constexpr int LDS_X = lds_elems<OX, Term::BKP>();
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wx = wave % Term::WX, wy = wave / Term::WX;
+    const T* lds_x = region;
+    const T* lds_y = region + LDS_X;
+    Acc acc[TY][TX];
+#pragma unroll
+    for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+        for (int tj = 0; tj < TX; tj++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++) acc[ti][tj][r] = (T)0;
+#pragma unroll
+    for (int k4 = 0; k4 < Term::BKP / KSTEP; k4++) {
+        const int kk = k4 * KSTEP + lane / MT;
+        T a[TY], b[TX];
+#pragma unroll
+        for (int ti = 0; ti < TY; ti++) a[ti] = lds_y[lds_addr<OY>(kk, (wy * TY + ti) * MT + lane % MT)];
+#pragma unroll
+        for (int tj = 0; tj < TX; tj++) b[tj] = lds_x[lds_addr<OX>(kk, (wx * TX + tj) * MT + lane % MT)];
+#pragma unroll
+        for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+            for (int tj = 0; tj < TX; tj++) acc[ti][tj] = MM::mma(a[ti], b[tj], acc[ti][tj]);
+    }
+    TermGeom<Term> g;
+    term_setup<Term>(g, ga, ta, origin);
+    int cx[TX][1], cy[TY][NREG];
+    c_tile_offsets<Term, FULL, false, true>(lane, wx, wy, g.rem, g.d, cx, cy);
+    constexpr bool ALL = FULL && Term::BXP == Term::BX && Term::BYP == Term::BY;     // no lane holds a position outside the tile
+#pragma unroll
+    for (int ti = 0; ti < TY; ti++)
+#pragma unroll
+        for (int tj = 0; tj < TX; tj++)
+#pragma unroll
+            for (int r = 0; r < NREG; r++)
+                if (ALL || (cx[tj][0] >= 0 && cy[ti][r] >= 0)) lds_accumulate(lds_c + cx[tj][0] + cy[ti][r], (T)acc[ti][tj][r]);
+}
+
+template <class... Terms> struct TermList {};
+template <int I, class First, class... Rest> struct TermAt { typedef typename TermAt<I - 1, Rest...>::type type; };
+template <class First, class... Rest> struct TermAt<0, First, Rest...> { typedef First type; };
+constexpr int tc_max_of() { return 0; }
+template <class... R> constexpr int tc_max_of(int a, R... r) { return a > tc_max_of(r...) ? a : tc_max_of(r...); }
+
+// NREGION = 2: as above.  NREGION = 1: one operand region; the slices of term t + 1 wait in registers until everybody
+// has finished term t (a second barrier per term), which halves the operand LDS and so lets twice as many workgroups
+// share a CU -- the kernel is bound by latency, not by bandwidth, so resident wavefronts are what it wants.
+// FULL: every extent is a whole number of tiles, so nothing is predicated.
+template <int NREGION, bool FULL, class G, class... Terms>
+__global__ __launch_bounds__(G::NT)
+void tc_group_pipe_kernel(typename G::T* __restrict__ C, const TcGroupArgs<(int)sizeof...(Terms)> ga)
+{
+    typedef typename G::T T;
+    constexpr int N = (int)sizeof...(Terms);
+    constexpr int NT = G::NT, VOL = G::TILE_VOL;
+    constexpr int MAXX = tc_max_of(PipeSlots<Terms, FULL>::X...), MAXY = tc_max_of(PipeSlots<Terms, FULL>::Y...);
+    T* const lds_c = (T*)tc_dynamic_lds;
+    T* const lds_ops = lds_c + VOL;                          // two regions of G::LDS_OPS elements
+    const int tid = threadIdx.x;
+
+    int origin[G::NIDX];
+#pragma unroll
+    for (int i = 0; i < G::NIDX; i++) origin[i] = 0;
+    int64_t baseC = 0;
+    {
+        // tiles in the order of their origins in C's memory: the tiles in flight chip-wide form one compact window
+        unsigned b = blockIdx.x;
+#pragma unroll
+        for (int j = 0; j < G::CR; j++) {
+            const int id = G::c_id(j);
+            const unsigned nb = (unsigned)ga.nblk[id];
+            origin[id] = (int)(b % nb) * G::c_tile(j);
+            b /= nb;
+            baseC += (int64_t)origin[id] * ga.sC[id];
+        }
+    }
+    T* __restrict__ Cb = C + uniform64(baseC);
+    auto c_element = [&](unsigned q, unsigned& off) -> bool {
+        bool ok = true;
+        off = 0;
+#pragma unroll
+        for (int j = 0; j < G::CR; j++) {
+            const unsigned t = (unsigned)G::c_tile(j);
+            const int c = (int)(q % t);
+            q /= t;
+            const int id = G::c_id(j);
+            off += (unsigned)c * (unsigned)ga.sC[id];
+            if (!FULL) ok = ok && (origin[id] + c < ga.ext[id]);
+        }
+        return ok;
+    };
+    // whole tiles: CV consecutive elements of C's fastest index per lane and access (C's fastest stride is 1)
+    constexpr int CV = (FULL && G::c_tile(0) % (16 / (int)sizeof(T)) == 0 && VOL % (NT * (16 / (int)sizeof(T))) == 0) ? 16 / (int)sizeof(T) : 1;
+    typedef T TCV __attribute__((ext_vector_type(CV), aligned(sizeof(T))));
+    typedef T TLV __attribute__((ext_vector_type(CV)));
+    constexpr int NEL = (VOL / CV + NT - 1) / NT;
+    T px[2][MAXX], py[2][MAXY];
+    {
+        // the first two terms' slices are requested before the C tile: they come from L2, the tile from HBM
+        typedef typename TermAt<0, Terms...>::type Term0;
+        typedef typename TermAt<(N > 1 ? 1 : 0), Terms...>::type Term1;
+        group_load<Term0, FULL, MAXX, MAXY>(px[0], py[0], ga, ga.term[0], origin, tid);
+        if constexpr (N > 1) group_load<Term1, FULL, MAXX, MAXY>(px[1], py[1], ga, ga.term[1], origin, tid);
+        TLV v[NEL];
+#pragma unroll
+        for (int i = 0; i < NEL; i++) {
+            const unsigned q = (unsigned)(tid + i * NT) * CV;
+            unsigned off;
+#pragma unroll
+            for (int e = 0; e < CV; e++) v[i][e] = (T)0;
+            if ((VOL % (NT * CV) == 0 || q < (unsigned)VOL) && c_element(q, off)) {
+                const TCV w = __builtin_nontemporal_load((const TCV*)(Cb + off));
+#pragma unroll
+                for (int e = 0; e < CV; e++) v[i][e] = w[e];
+            }
+        }
+        group_store<G, Term0, FULL, MAXX, MAXY>(px[0], py[0], lds_ops, ga, ga.term[0], origin, tid);
+#pragma unroll
+        for (int i = 0; i < NEL; i++) {
+            const unsigned q = (unsigned)(tid + i * NT) * CV;
+            if (VOL % (NT * CV) == 0 || q < (unsigned)VOL) *(TLV*)(lds_c + q) = v[i];
+        }
+        __syncthreads();
+    }
+    static_for<N>([&](auto tt) {
+        constexpr int t = decltype(tt)::value;
+        typedef typename TermAt<t, Terms...>::type Term;
+        typedef typename TermAt<(t + 1 < N ? t + 1 : t), Terms...>::type Next;
+        typedef typename TermAt<(t + 2 < N ? t + 2 : t), Terms...>::type Far;
+        if constexpr (t + 2 < N) group_load<Far, FULL, MAXX, MAXY>(px[t & 1], py[t & 1], ga, ga.term[t + 2], origin, tid);
+        group_contract<G, Term, FULL>(lds_c, lds_ops + (NREGION == 2 ? (t & 1) : 0) * G::LDS_OPS, ga, ga.term[t], origin, tid);
+        if constexpr (NREGION == 1 && t + 1 < N) __syncthreads();          // everybody is done reading the one region
+        if constexpr (t + 1 < N) group_store<G, Next, FULL, MAXX, MAXY>(px[(t + 1) & 1], py[(t + 1) & 1], lds_ops + (NREGION == 2 ? ((t + 1) & 1) : 0) * G::LDS_OPS, ga, ga.term[t + 1], origin, tid);
+        __syncthreads();
+    });
+#pragma unroll
+    for (int i = 0; i < NEL; i++) {
+        const unsigned q = (unsigned)(tid + i * NT) * CV;
+        unsigned off;
+        if ((VOL % (NT * CV) == 0 || q < (unsigned)VOL) && c_element(q, off)) {
+            const TLV w = *(const TLV*)(lds_c + q);
+            TCV o;
+#pragma unroll
+            for (int e = 0; e < CV; e++) o[e] = w[e];
+            __builtin_nontemporal_store(o, (TCV*)(Cb + off));
+        }
     }
 }
 
@@ -317,7 +554,46 @@ int tc_group_run(const int* sizes, void* C, const void* const* inputs, const int
     if (too_far) return tc_fail(TC_ERR_TOO_LARGE, "a tile of this mapping spans 4 GB or more of a tensor (byte offsets inside a tile are 32-bit)");
 
     tc_clear_hip_error();
-    hipLaunchKernelGGL((tc_group_kernel<G, Terms...>), dim3((unsigned)grid), dim3(G::NT), 0, stream, (T*)C, ga);
+    // every term enabled, every contracted range within one K block: the pipelined kernel
+    bool pipe = true;
+    for (int i = 0; i < N; i++) pipe = pipe && ga.term[i].enabled;
+    auto one_kb = [&](auto term) {
+        typedef decltype(term) Term;
+        for (int i = 0; i < Term::NK; i++) if (sizes[Term::k_id(i)] > Term::k_tile(i)) pipe = false;
+    };
+    (one_kb(Terms()), ...);
+    // whole tiles everywhere (the contracted extents then equal their tiles): the variant without predicates
+    bool full = true;
+    for (int j = 0; j < G::CR; j++) if (sizes[G::c_id(j)] % G::c_tile(j)) full = false;
+    auto whole_k = [&](auto term) {
+        typedef decltype(term) Term;
+        for (int i = 0; i < Term::NK; i++) if (sizes[Term::k_id(i)] != Term::k_tile(i)) full = false;
+    };
+    (whole_k(Terms()), ...);
+    constexpr int NREGION = G::NREGION > 0 ? G::NREGION : 1;
+    if (G::NREGION == 0) pipe = false;                 // nr=0: the kernel with one load-store-contract pass per term
+    constexpr size_t pipe_lds = sizeof(T) * ((size_t)G::TILE_VOL + NREGION * (size_t)G::LDS_OPS);
+    constexpr size_t serial_lds = sizeof(T) * ((size_t)G::TILE_VOL + (size_t)G::LDS_OPS);
+    static_assert(serial_lds <= 160 * 1024, "the C tile and one operand region exceed the LDS of a CU");
+    if (pipe_lds > 160 * 1024) pipe = false;
+    if (pipe_lds > 65536 || serial_lds > 65536) {
+        // more than the 64 KB a kernel may use unasked: raise the limit once per device
+        static std::atomic<bool> configured[64];
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return tc_fail(TC_ERR_LAUNCH, "no current device for the fused group kernel");
+        if (!configured[dev].load(std::memory_order_acquire)) {
+            bool ok = hipFuncSetAttribute((const void*)&tc_group_kernel<G, Terms...>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)serial_lds) == hipSuccess;
+            if (pipe_lds <= 160 * 1024) {
+                ok = ok && hipFuncSetAttribute((const void*)&tc_group_pipe_kernel<NREGION, false, G, Terms...>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pipe_lds) == hipSuccess;
+                ok = ok && hipFuncSetAttribute((const void*)&tc_group_pipe_kernel<NREGION, true, G, Terms...>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pipe_lds) == hipSuccess;
+            }
+            if (!ok) { (void)hipGetLastError(); return tc_fail(TC_ERR_LAUNCH, "the fused group kernel's LDS size was refused"); }
+            configured[dev].store(true, std::memory_order_release);
+        }
+    }
+    if (pipe && full) hipLaunchKernelGGL((tc_group_pipe_kernel<NREGION, true, G, Terms...>), dim3((unsigned)grid), dim3(G::NT), pipe_lds, stream, (T*)C, ga);
+    else if (pipe)    hipLaunchKernelGGL((tc_group_pipe_kernel<NREGION, false, G, Terms...>), dim3((unsigned)grid), dim3(G::NT), pipe_lds, stream, (T*)C, ga);
+    else              hipLaunchKernelGGL((tc_group_kernel<G, Terms...>), dim3((unsigned)grid), dim3(G::NT), serial_lds, stream, (T*)C, ga);
     return tc_check_launch("fused group kernel launch failed");
 }
 

@@ -75,6 +75,7 @@ static bool term_mapping(const Contraction& c, DType t, const ArchGfx950& arch, 
     auto fvi = [](const std::vector<int>& v) { return v.empty() ? -1 : v[0]; };
     m.layx = (!m.k_ids.empty() && m.k_ids[0] == fvi(xop) && m.k_tiles[0] >= 4) ? 1 : 0;
     m.layy = (!m.k_ids.empty() && m.k_ids[0] == fvi(yop) && m.k_tiles[0] >= 4) ? 1 : 0;
+    m.VL = 1;                              // 16-byte slice loads wherever a call's tiles are whole (the pipelined kernel's variant without predicates)
     finish_geometry(c, t, m);
     if (!check_mapping(c, t, arch, m, err)) return false;
     return true;
@@ -111,7 +112,7 @@ bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& a
     auto evaluate = [&](const std::vector<int>& tile, std::vector<Mapping>& maps, double& score) -> bool {
         long long vol = 1;
         for (int v : tile) vol *= v;
-        if (vol > vol_max) { why = "the tile of the output exceeds 32 KB"; return false; }
+        if (vol > 2 * vol_max) { why = "the tile of the output exceeds 64 KB"; return false; }
         maps.assign(cs.size(), Mapping());
         double mfma_eff = 0, op_eff = 0;
         int lds_ops = 0;
@@ -119,7 +120,8 @@ bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& a
             std::string e;
             if (!term_mapping(cs[k], t, arch, tile, g.NW, g.k_room, maps[k], e)) { why = "term " + std::to_string(k + 1) + ": " + e; return false; }
             const Mapping& m = maps[k];
-            if (m.lds_bytes > 32768) { why = "term " + std::to_string(k + 1) + ": input slices exceed 32 KB"; return false; }
+            if (m.lds_bytes > 65536) { why = "term " + std::to_string(k + 1) + ": input slices exceed 64 KB"; return false; }
+            if (vol * s + m.lds_bytes > 160 * 1024) { why = "term " + std::to_string(k + 1) + ": the tile of the output and the input slices exceed the 160 KB of LDS"; return false; }
             lds_ops = std::max(lds_ops, m.lds_bytes);
             mfma_eff += (double)(m.BX * m.BY) / (double)(m.BXP * m.BYP);
             for (int side = 0; side < 2; side++) {
@@ -139,7 +141,7 @@ bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& a
         double run = 1;
         for (int j = 0; j < CR; j++) { run *= tile[j]; if (tile[j] != c0.indices[c0.out_idx[j]].rep_size) break; }
         const double run_eff = std::min(1.0, 0.75 + 0.25 * std::log2(std::max(1.0, run * s / 128.0)) / 4.0);
-        score = c_eff * (0.5 + 0.5 * op_eff) * (0.3 + 0.7 * mfma_eff) * (0.5 + 0.5 * (double)vol / vol_max) * run_eff;
+        score = c_eff * (0.5 + 0.5 * op_eff) * (0.3 + 0.7 * mfma_eff) * (0.5 + 0.5 * std::min(1.0, (double)vol / vol_max)) * run_eff;
         (void)lds_ops;
         return true;
     };
@@ -155,7 +157,8 @@ bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& a
             if (field.compare(0, 3, "ct=") == 0) ct_spec = field.substr(3);
             else if (field.compare(0, 3, "kt=") == 0) g.k_room = std::max(4, std::min(64, atoi(field.c_str() + 3)));
             else if (field.compare(0, 3, "nw=") == 0) g.NW = std::max(1, std::min(8, atoi(field.c_str() + 3)));
-            else { err = "group mapping spec: fields are ct=<tile>,... kt=<n> nw=<n>"; return false; }
+            else if (field.compare(0, 3, "nr=") == 0) g.nregion = std::max(0, std::min(2, atoi(field.c_str() + 3)));
+            else { err = "group mapping spec: fields are ct=<tile>,... kt=<n> nw=<n> nr=<0|1|2>"; return false; }
         }
     }
     if (!ct_spec.empty()) {
@@ -205,7 +208,7 @@ std::string group_json(const GroupPlan& g)
     for (size_t j = 0; j < g.c_tile.size(); j++) o << (j ? ", " : "") << g.c_tile[j];
     o << "], \"threads\": " << 64 * g.NW << ", \"lds_bytes\": " << (g.vol + g.lds_ops) * esize(g.t) << ", \"spec\": \"ct=";
     for (size_t j = 0; j < g.c_tile.size(); j++) o << (j ? "," : "") << g.c_tile[j];
-    o << ";kt=" << g.k_room << ";nw=" << g.NW << "\", \"terms\": [";
+    o << ";kt=" << g.k_room << ";nw=" << g.NW << ";nr=" << g.nregion << "\", \"terms\": [";
     for (size_t k = 0; k < g.terms.size(); k++)
         o << (k ? ", " : "") << "{\"text\": \"" << c_escape(g.terms[k].text) << "\", \"mapping\": " << mapping_json(g.terms[k], g.t, g.maps[k]) << "}";
     o << "]}";
@@ -230,7 +233,7 @@ std::string emit_group_source(const GroupPlan& g, const std::string& unique_name
     };
     o << "struct G {\n    typedef " << T << " T;\n";
     o << "    static constexpr int NIDX = " << c0.n_idx() << ", CR = " << c0.out_idx.size() << ", NTERM = " << N << ", NT = " << 64 * g.NW
-      << ", TILE_VOL = " << g.vol << ", LDS_OPS = " << g.lds_ops << ";\n";
+      << ", TILE_VOL = " << g.vol << ", LDS_OPS = " << g.lds_ops << ", NREGION = " << g.nregion << ";\n";
     table("c_id", c0.out_idx);
     table("c_tile", g.c_tile);
     o << "};\n";

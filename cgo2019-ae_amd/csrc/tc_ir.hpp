@@ -126,6 +126,7 @@ struct GroupPlan {
     std::vector<Mapping> maps;        // per term: roles and tiles derived from c_tile
     int NW = 4;                       // wavefronts per workgroup
     int k_room = 32;                  // contracted depth per K block
+    int nregion = 1;                  // operand regions in LDS of the pipelined kernel (spec nr=): 1 = more workgroups per CU, 2 = one barrier per term
     int vol = 0, lds_ops = 0;         // elements of the C tile; elements of the largest pair of operand slices
 };
 // spec: empty (search) or fields "ct=<tile>,<tile>,..." (one per output index), "kt=<K depth>", "nw=<wavefronts>" joined by ';'
