@@ -37,7 +37,7 @@ def test_group_plan_shares_one_tile_and_gives_each_term_its_own_roles():
     assert j["out_idx"] == ["h3", "h2", "h1", "p6", "p5", "p4"] and j["sum_idx"] == ["p7"]
     tile = dict(zip(j["out_idx"], j["c_tile"]))
     vol = int(np.prod(j["c_tile"]))
-    assert 256 <= vol * 8 <= 32768 and j["lds_bytes"] <= 65536
+    assert 256 <= vol * 8 <= 32768 and j["lds_bytes"] <= 160 * 1024          # dynamic LDS: the CU's 160 KB is the limit
     for term in j["terms"]:
         m = term["mapping"]
         # every output index is tiled exactly once, with the group's tile, on the side of the input that holds it
@@ -52,9 +52,12 @@ def test_group_plan_shares_one_tile_and_gives_each_term_its_own_roles():
 
 def test_group_tile_spec_and_rejections(tmp_path):
     rc, j = plan_json(FUSED, spec="ct=16,2,2,4,2,2")
-    assert rc == 0 and j["c_tile"] == [16, 2, 2, 4, 2, 2] and j["spec"] == "ct=16,2,2,4,2,2;kt=32;nw=4"
+    assert rc == 0 and j["c_tile"] == [16, 2, 2, 4, 2, 2] and j["spec"] == "ct=16,2,2,4,2,2;kt=32;nw=4;nr=1"
     rc, j = plan_json(FUSED, spec="ct=16,4,4,2,2,2;kt=8;nw=8")                 # K depth per block, wavefronts per workgroup
     assert rc == 0 and j["threads"] == 512 and all(t["mapping"]["block_tile"][2] == 8 for t in j["terms"])
+    for nr in (0, 1, 2):                                               # operand regions of the pipelined kernel; 0 = the per-term kernel
+        rc, j = plan_json(FUSED, spec="ct=16,4,4,2,2,2;kt=16;nw=4;nr=%d" % nr)
+        assert rc == 0 and j["spec"].endswith(";nr=%d" % nr)
     rc, err = plan_json(FUSED, spec="tile=3")
     assert rc == 3 and "fields are" in err
     rc, err = plan_json(FUSED, spec="ct=16,16,16,16,1,1")              # 64 K elements of C: does not fit
@@ -132,7 +135,7 @@ def group():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["fused_sd2_f64", "fused_sd1_f32"])
+@pytest.mark.parametrize("name", ["fused_sd2_f64", "fused_sd1_f32", "var_fused_sd2_two_regions_f64", "var_fused_sd1_per_term_pass_f32"])
 @pytest.mark.parametrize("sizes", [[5, 3, 7, 6, 2, 9, 4], [16, 4, 4, 2, 2, 2, 16], [17, 5, 6, 3, 4, 3, 19], [1, 1, 1, 1, 1, 1, 1],
                                    [32, 8, 4, 4, 4, 2, 24], [16, 16, 16, 16, 8, 8, 16]])
 def test_fused_group_matches_the_terms_applied_one_by_one(name, sizes, tools, oracle):
