@@ -236,6 +236,14 @@ bool check_mapping(const Contraction& c, DType t, const ArchGfx950& arch, const 
     return true;
 }
 
+// LDS of the streaming kernel: the resident panel over all K blocks and two slices of the other side
+static long long stream_lds_bytes(DType t, const Mapping& m, long long nkb)
+{
+    const long long lds_x = (m.layx == 0 ? (long long)m.BKP * m.ldx : (long long)m.BXP * m.ldx);
+    const long long lds_y = (m.layy == 0 ? (long long)m.BKP * m.ldy : (long long)m.BYP * m.ldy);
+    return (long long)esize(t) * (m.SRES ? nkb * lds_y + 2 * lds_x : nkb * lds_x + 2 * lds_y);
+}
+
 void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& m)
 {
     const MiInfo mi = mi_info(m.MI);
@@ -307,7 +315,20 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
         m.CLDS = (m.clds_forced == 1 && possible) ? 1 : 0;
         if (m.CLDS && m.ntc_forced < 0) m.NTC = whole_lines ? 3 : 0;
     }
-    const double c_hbm_eff = m.CLDS ? 1.0 : std::min(1.0, chunk * s / 128.0);
+    // 128-byte lines a contiguous chunk of the tile touches, relative to the bytes it holds: chunks start at multiples
+    // of g bytes (their own size, and C's row pitch when a chunk is part of a row), so a chunk touches
+    // bytes / 128 + 1 - gcd(g, 128) / 128 lines on average; the lines it only partly owns are shared with a neighbouring
+    // tile and move twice (config 2: 128-byte chunks at a 576-byte row pitch measured 196 us, 192-byte chunks 118,
+    // whole 1152-byte chunks 98)
+    double c_hbm_eff;
+    {
+        const long long chunk_b = (long long)(chunk * s), row_b = (long long)(ext(c.out_idx[0]) * s);
+        const bool within_row = tile_of(c.out_idx[0]) != c.indices[c.out_idx[0]].rep_size;
+        long long g = within_row ? std::__gcd(chunk_b, row_b) : chunk_b;
+        g = std::__gcd(g, 128LL);
+        const double lines = (double)chunk_b / 128.0 + 1.0 - (double)g / 128.0;
+        c_hbm_eff = ((double)chunk_b / 128.0) / lines;
+    }
     // address span of the block's C tile relative to its volume: compact tiles keep DRAM pages and
     // TLB entries busy with fewer blocks (measured: tiling the Y side in C's own index order beats
     // the operand's order by 20-40% on the 6-D contractions)
@@ -329,6 +350,7 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const int slots = (int)(std::ceil((double)m.BK * m.BX / (64.0 * W)) + std::ceil((double)m.BK * m.BY / (64.0 * W)));
     int regs = acc_regs + 40 + slots * r4 + (m.TX + m.TY * mi.NREG) + (m.TX + m.TY) * r4;
     if (nkb > 1) regs += 2 * slots;
+    if (m.STREAM > 0) regs += acc_regs;                 // the streaming kernel holds the next tile's C values next to the accumulators
     // prefetch depth: one K block ahead unless a mapping spec asks for more (pd=); each extra stage
     // holds one slice share in registers, and on the shapes measured so far the registers were worth
     // more as a resident wavefront
@@ -339,7 +361,8 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const double spill_penalty = regs > reg_cap ? 1.0 + 2.0 * (double)(regs - reg_cap) / reg_cap : 1.0;
     int waves_per_simd = std::max(1, std::min(8, arch.vgpr_per_lane / std::max(regs, 64)));
     const bool two_stage = nkb > 1 && (2 * m.lds_bytes <= arch.lds_bytes_per_block || (m.DBUF && 2 * m.lds_bytes <= arch.lds_bytes_per_cu));
-    const int lds_block = std::max(m.lds_bytes * (two_stage ? 2 : 1), m.CLDS ? (int)(m.BX * m.BY * s) : 0);
+    int lds_block = std::max(m.lds_bytes * (two_stage ? 2 : 1), m.CLDS ? (int)(m.BX * m.BY * s) : 0);
+    if (m.STREAM > 0) lds_block = (int)std::min<long long>(arch.lds_bytes_per_cu, stream_lds_bytes(t, m, m.STREAM));
     int r = std::min(arch.lds_bytes_per_cu / std::max(lds_block, 1), arch.max_waves_per_cu / W);
     r = std::min(r, std::max(1, waves_per_simd * arch.simd_per_cu / W));
     r = std::max(r, 1);
@@ -367,8 +390,17 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
         while (j + 1 < op.size() && tile_of(op[j]) == c.indices[op[j]].rep_size) { rn *= tile_of(op[j + 1]); j++; }
         return std::min(1.0, rn * s / 128.0);
     };
-    const double stage_x = (double)nblocks * nkb * m.BK * m.BX * s;
-    const double stage_y = (double)nblocks * nkb * m.BK * m.BY * s;
+    double stage_x = (double)nblocks * nkb * m.BK * m.BX * s;
+    double stage_y = (double)nblocks * nkb * m.BK * m.BY * s;
+    if (m.STREAM > 0) {
+        // panel-resident streaming kernel: a workgroup fetches the resident side once for its whole run of tiles,
+        // and its reads of the next tile's C are in flight while the current one is contracted, so that the
+        // memory pipe does not wait for co-resident workgroups in other phases (measured 0.55-0.75 of the HBM
+        // peak with ONE workgroup per CU, where the per-tile kernel needs three)
+        const double wgs = (double)std::min<long long>(nblocks, (long long)arch.n_cu * std::max(1, m.blocks_per_cu));
+        (m.SRES ? stage_y : stage_x) *= wgs / (double)nblocks;
+        m.t_hbm *= occ_eff / std::min(0.95, 0.55 + 0.05 * r * W);
+    }
     m.t_l2 = stage_x / (arch.l2_bytes_per_s * op_eff(xop)) + stage_y / (arch.l2_bytes_per_s * op_eff(yop));
 
     // ---- matrix cores: wavefronts of the resident blocks spread over 4 SIMDs (9 wavefronts leave
@@ -387,7 +419,10 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const double t_overhead = (double)nblocks * nkb * W * (250.0 + 10.0 * slots) / simd_hz;
     // an LDS-fed MFMA loop needs co-resident wavefronts to cover LDS and MFMA latency: measured 68 % of
     // peak with one wavefront per SIMD, 84 % with two, little more beyond
-    const double mfma_occ = waves_simd >= 3.0 ? 0.92 : waves_simd >= 2.0 ? 0.84 : 0.68;
+    // (the wavefronts of ONE workgroup meet at every barrier and so stall together: what counts is the number of
+    // workgroups on the CU -- twelve wavefronts of one workgroup measured 64 % on config 3, where two workgroups
+    // of four reached 77 % with a second K block requested ahead)
+    const double mfma_occ = std::min(0.95, (r >= 3 ? 0.92 : r == 2 ? 0.84 : 0.70) + (m.PD >= 2 ? 0.05 : 0.0));
     m.t_mfma = (n_mfma * mi.cycles / simd_hz / mfma_occ + t_overhead) / simd_busy;
 
     const double lds_reads = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * W * (m.TX + m.TY) * 64.0 * s;
@@ -402,10 +437,94 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     double mx = t_l1, sum = t_l1;
     for (double p : parts) { mx = std::max(mx, p); sum += p; }
     // the slowest pipe sets the pace; the others overlap imperfectly
-    m.cost = (mx + 0.15 * (sum - mx)) * spill_penalty / std::max(m.tail_eff, 0.05) + 2.0e-6;
+    // (where HBM sets the pace the slice traffic weighs more than the rest: the slices come through the same L2 and
+    // fabric as C, and the mappings measured best on the 6-D shapes were those with the least of it among near-equal
+    // HBM terms)
+    m.cost = (mx + 0.15 * (sum - mx) + (std::max(m.t_hbm, m.t_l2) >= mx ? 0.25 * std::min(m.t_l2, m.t_hbm) : 0.0)) * spill_penalty / std::max(m.tail_eff, 0.05) + 2.0e-6;
+    // the streaming kernel must win clearly: on the 6-D shapes it measured level with the per-tile kernel for most
+    // index orders and a third slower for some, which nothing above tells apart
+    if (m.STREAM > 0) m.cost *= 1.05;
     // a repacked input is read and written once more by a kernel of its own, which the contraction waits for
     if (m.RPX) m.cost += 2.0 * nX * s / bw + 4.0e-6;
     if (m.RPY) m.cost += 2.0 * nY * s / bw + 4.0e-6;
+}
+
+static bool plan_stream(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& m, std::string& err);
+
+static long long k_blocks(const Contraction& c, const Mapping& m)
+{
+    long long nkb = 1;
+    for (size_t i = 0; i < m.k_ids.size(); i++) nkb *= ceil_div(c.indices[m.k_ids[i]].rep_size, m.k_tiles[i]);
+    return nkb;
+}
+
+// 16-byte slice loads (vl=) for the inputs whose tile along their fastest index spans at least half a line
+static int vector_sides(const Contraction& c, DType t, const Mapping& m)
+{
+    auto tile_of = [&](int id) -> int {
+        int p;
+        if ((p = pos_in(m.x_ids, id)) >= 0) return m.x_tiles[p];
+        if ((p = pos_in(m.y_ids, id)) >= 0) return m.y_tiles[p];
+        if ((p = pos_in(m.k_ids, id)) >= 0) return m.k_tiles[p];
+        return 1;
+    };
+    const std::vector<int> xop = operand_order(c, m, true), yop = operand_order(c, m, false);
+    const bool vx = !xop.empty() && tile_of(xop[0]) * esize(t) >= 64, vy = !yop.empty() && tile_of(yop[0]) * esize(t) >= 64;
+    return vx && vy ? 1 : vx ? 2 : vy ? 3 : 0;
+}
+
+// Options that the cost terms do not separate, set the way they measured best on the part.  (A mapping spec sets
+// them itself; these rules only act on the mappings the pass enumerates.)
+//   One K block (the many-index shapes whose cost is the traffic of C): tiles handed out in the order of their
+//   origins in C's memory, -7 to -12 % on the 6-D shapes of the benchmark set; 16-byte slice loads where a tile
+//   allows, -1 to -2 %; C through LDS when C's rows are not whole 128-byte lines (96-byte fp32 rows, 192-byte
+//   fp64 rows: -5 % and -3 to -5 %), not otherwise (+12 % on 128-byte rows).
+static void measured_rules(const Contraction& c, DType t, Mapping& m)
+{
+    if (k_blocks(c, m) != 1 || m.SK > 1) return;
+    m.TORD = 1;
+    m.VL = 1;
+    const long long row = (long long)m.x_tiles[0] * esize(t);
+    if (row % 128 != 0 && row % 16 == 0) m.clds_forced = 1;
+}
+
+// The streaming kernel for an enumerated mapping: depth 3 for three K blocks, else 2; C non-temporal; runs of the
+// workgroups interleaved (-1 to -4 % wherever it was measured); the resident panel loaded behind the first tile when
+// it is larger than 64 KB (config 2: -4 %).
+static bool stream_variant(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& m)
+{
+    const long long nkb = k_blocks(c, m);
+    // three K blocks or more: with two, the kernel measured level with the per-tile kernel at best (config 4 with 16s,
+    // some 6-D shapes) and a third to two thirds slower on others (config 4, config 5 #9), which nothing here tells apart
+    if (nkb < 3 || nkb > 64 || m.SK > 1) return false;
+    if (t != DType::F64) return false;       // fp32: its one measured win had two K blocks; the six-index fp32 shape ran 1.7 to 2 times slower with it
+    // every measured win of this kernel had eight or more wavefronts with at most three accumulator tiles each (its one
+    // workgroup per CU is all that hides the memory latency; two wavefronts with 18 tiles each ran at half the
+    // per-tile kernel's speed on config 4)
+    if (m.WX * m.WY < 8 || m.TX * m.TY > 3) return false;
+    // ... and contiguous chunks of C made of whole 128-byte lines, which its non-temporal accesses need (on partial
+    // lines they defeat write combining: +35 % on 96-byte fp32 rows)
+    {
+        long long chunk = esize(t);
+        for (int id : c.out_idx) {
+            int p, tl = 1;
+            if ((p = pos_in(m.x_ids, id)) >= 0) tl = m.x_tiles[p];
+            else if ((p = pos_in(m.y_ids, id)) >= 0) tl = m.y_tiles[p];
+            chunk *= tl;
+            if (tl != c.indices[id].rep_size) break;
+        }
+        if (chunk % 128) return false;
+    }
+    m.st_forced = nkb == 3 ? 3 : nkb % 2 == 0 ? 2 : nkb % 3 == 0 ? 3 : 0;
+    if (m.st_forced == 0) return false;
+    std::string err;
+    if (!plan_stream(c, t, arch, m, err)) return false;
+    m.ntc_forced = 3;
+    m.SIL = 1;
+    const long long panel = (long long)esize(t) * nkb * (m.layx == 0 ? (long long)m.BKP * m.ldx : (long long)m.BXP * m.ldx);
+    m.SOV = panel > 65536 ? 1 : 0;
+    m.VL = vector_sides(c, t, m);
+    return true;
 }
 
 static void wave_layouts(int nx, int ny, int max_acc_tiles, std::vector<std::array<int, 4>>& out)
@@ -517,8 +636,14 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
                         finish_geometry(c, t, m);
                         std::string err;
                         if (!check_mapping(c, t, arch, m, err)) continue;
+                        measured_rules(c, t, m);
                         cost_model(c, t, arch, m);
                         out.push_back(m);
+                        // the streaming kernel wherever it can run with this tile
+                        {
+                            Mapping mv = m;
+                            if (stream_variant(c, t, arch, mv)) { cost_model(c, t, arch, mv); out.push_back(mv); }
+                        }
                         // few output tiles and a long K loop: also try splitting K over 2, 4, 8 workgroups
                         const long long tiles = m.n_blocks;
                         const int ksteps = m.steps_main_loop;
@@ -575,9 +700,7 @@ static bool plan_stream(const Contraction& c, DType t, const ArchGfx950& arch, M
         err = "streaming kernel (st=): needs 2..64 K blocks and a prefetch depth that divides their number (K blocks here: " + std::to_string(nkb) + ")";
         return false;
     }
-    const long long lds_x = (m.layx == 0 ? (long long)m.BKP * m.ldx : (long long)m.BXP * m.ldx);
-    const long long lds_y = (m.layy == 0 ? (long long)m.BKP * m.ldy : (long long)m.BYP * m.ldy);
-    const long long bytes = (long long)esize(t) * (m.SRES ? nkb * lds_y + 2 * lds_x : nkb * lds_x + 2 * lds_y);
+    const long long bytes = stream_lds_bytes(t, m, nkb);
     if (bytes > arch.lds_bytes_per_cu) {
         err = "streaming kernel (st=): the resident panel needs " + std::to_string(bytes) + " bytes of LDS";
         return false;
