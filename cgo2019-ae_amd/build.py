@@ -153,6 +153,26 @@ def emit_and_compile(entry):
     return name
 
 
+def model_name(name):
+    return "model_" + name
+
+
+def emit_and_compile_model_pick(entry):
+    """The same expression compiled from the mapping pass's FIRST pick: no mapping spec, no tuned table.  These
+    objects (lib/model_<name>.so, benchmark configurations only) exist to measure the mapping pass on its own against
+    the tuned objects."""
+    name = model_name(entry["name"])
+    hip = os.path.join(GEN, name + ".hip")
+    run([os.path.join(BIN, "cogent_gen"), name, os.path.join(EXPR, entry["file"]), "-1", "-1", entry["dtype"],
+         "-o", hip, "--name", name, "--json"])
+    run(["hipcc"] + HIPCC_FLAGS + ["-o", os.path.join(LIB, name + ".so"), hip])
+    return name
+
+
+def benchmark_configs():
+    return [e for e in manifest() if e["name"].startswith("cfg")]
+
+
 def build_driver():
     run(["hipcc"] + HIPCC_FLAGS + ["-o", os.path.join(LIB, "libcogent_driver.so"),
                                    os.path.join(CSRC, "tc_driver.cpp"), "-ldl"])
@@ -164,6 +184,7 @@ def build_all(jobs=8, only=None):
     entries = [e for e in manifest() + group_manifest() if only is None or e["name"] in only]
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         futs = [ex.submit(emit_and_compile, e) for e in entries]
+        futs += [ex.submit(emit_and_compile_model_pick, e) for e in benchmark_configs() if only is None or model_name(e["name"]) in only]
         futs.append(ex.submit(build_driver))
         for f in futs:
             f.result()

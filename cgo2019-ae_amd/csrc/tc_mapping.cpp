@@ -388,7 +388,12 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
         double rn = tile_of(op[0]);
         size_t j = 0;
         while (j + 1 < op.size() && tile_of(op[j]) == c.indices[op[j]].rep_size) { rn *= tile_of(op[j + 1]); j++; }
-        return std::min(1.0, rn * s / 128.0);
+        // an input of at most 2 MB stays in the L2 of every XCD (4 MB) and its lines are shared by neighbouring lanes and
+        // tiles: short runs then waste 32-byte requests, not 128-byte lines (config 4: 16-byte runs of a 1.3 MB input
+        // measured FASTER than 32-byte runs with twice the slice volume)
+        double total = s;
+        for (int id : op) total *= ext(id);
+        return std::min(1.0, rn * s / (total <= 2.0e6 ? 32.0 : 128.0));
     };
     double stage_x = (double)nblocks * nkb * m.BK * m.BX * s;
     double stage_y = (double)nblocks * nkb * m.BK * m.BY * s;
@@ -479,9 +484,12 @@ static int vector_sides(const Contraction& c, DType t, const Mapping& m)
 //   origins in C's memory, -7 to -12 % on the 6-D shapes of the benchmark set; 16-byte slice loads where a tile
 //   allows, -1 to -2 %; C through LDS when C's rows are not whole 128-byte lines (96-byte fp32 rows, 192-byte
 //   fp64 rows: -5 % and -3 to -5 %), not otherwise (+12 % on 128-byte rows).
+//   Several K blocks: 16-byte slice loads for the inputs whose tile along their fastest index spans half a line or
+//   more (config 1: -5 %).
 static void measured_rules(const Contraction& c, DType t, Mapping& m)
 {
-    if (k_blocks(c, m) != 1 || m.SK > 1) return;
+    if (k_blocks(c, m) != 1) { m.VL = vector_sides(c, t, m); return; }
+    if (m.SK > 1) return;
     m.TORD = 1;
     m.VL = 1;
     const long long row = (long long)m.x_tiles[0] * esize(t);

@@ -122,8 +122,12 @@ def test_kernel_options_in_a_spec(tools):
     assert tools.plan(text, "DOUBLE", mapping_spec=base + ";cl=1").info["mapping"]["c_through_lds"] == 0   # 96x96x8 B > 64 KB
     # fp32 with a fastest tile that is a multiple of 4: swapped roles by default, sw=0 turns them off
     text4 = open(os.path.join(EXPR_DIR, "cfg4_16_f32.in")).read()
-    auto = tools.plan(text4, "FLOAT").info["mapping"]
+    auto = tools.plan(text4, "FLOAT", mapping_spec="x=0:16,2:16,4:1;y=1:16,3:2,5:1;k=6:16;w=4x1;t=4x2;mi=1").info["mapping"]
     assert auto["swapped_roles"] == 1 and auto["nontemporal_c"] == 0           # 64-byte rows: no whole lines per access
+    # the pass's own pick for this shape (one K block, rows that are not whole lines): C through LDS in memory order,
+    # whose tile is made of whole lines, tiles in C's memory order, 16-byte slice loads
+    pick = tools.plan(text4, "FLOAT").info["mapping"]
+    assert pick["c_through_lds"] == 1 and pick["tile_order_c_memory"] == 1 and pick["vector_slice_loads"] == 1 and pick["stream"][0] == 0
     off = tools.plan(text4, "FLOAT", mapping_spec=auto["spec"] + ";sw=0").info["mapping"]
     assert off["swapped_roles"] == 0
     # fp64 rows of 16 elements are whole aligned lines: non-temporal loads and stores
