@@ -5,8 +5,9 @@ oracle/Makefile compiles cogent/drivers/tccg/code_main_tccg_NN.c with its checke
 sd_t_d2_fusion_host_ of lib/tccg_NN_f64.so, and links.  The driver allocates host tensors, fills them
 with rand(), calls the entry point as it would call COGENT's generated code
 (cogent/drivers/tccg/code_main_tccg_01.c:69) and checks the result with ITS host loop and ITS
-tolerance (1e-8 absolute for fp64, 1e-5 for fp32; :135-157).  Skipped where the binaries were not
-built (the reference tree is needed to build them, not to run them).
+tolerance (1e-8 absolute for fp64, 1e-5 for fp32; :135-157).  The 18 CCSD(T) drivers (cogent/drivers/ccsd_t) are linked
+the same way against the single-term objects lib/ccsd_sd<d>_<k>_f64.so.  Skipped where the binaries were not built (the
+reference tree is needed to build them, not to run them).
 """
 import os
 import re
@@ -45,6 +46,14 @@ for _n in range(1, 49):
         CASES.append(("drv_tccg_%02d" % _n, RAGGED[:n_indices(_n)]))
 for _n in range(40, 49):
     CASES.append(("drv_float_tccg_%02d" % _n, RAGGED[:n_indices(_n)]))
+# ... and the 18 CCSD(T) drivers (cogent/drivers/ccsd_t/code_main_sd1_1.c .. sd2_9.c): each calls the single-term entry
+# point for its own term (code_main_sd2_1.c:112-114) and checks it with the one active line of its loop (tolerance 1e-4,
+# :611-625), against lib/ccsd_sd<d>_<k>_f64.so.  Their command line is seven extents and the register-transpose option.
+for _fam in ("sd1", "sd2"):
+    for _k in range(1, 10):
+        CASES.append(("drv_ccsd_%s_%d" % (_fam, _k), RAGGED + [1]))
+CASES.append(("drv_ccsd_sd1_1", []))                   # built-in extents: all 16
+CASES.append(("drv_ccsd_sd2_9", []))
 
 
 @pytest.mark.parametrize("binary,sizes", CASES, ids=["%s-%s" % (b, "x".join(map(str, s)) or "default") for b, s in CASES])
