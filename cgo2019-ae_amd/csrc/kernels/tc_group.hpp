@@ -488,6 +488,162 @@ void tc_group_pipe_kernel(typename G::T* __restrict__ C, const TcGroupArgs<(int)
     }
 }
 
+// Persistent form of the pipelined kernel for whole tiles: a workgroup takes tiles blockIdx.x, + gridDim.x, ... and the
+// pipeline of the terms runs ACROSS tile boundaries -- during the last two terms of a tile the slices of the next
+// tile's first two terms are requested, during the last term its C tile, so that no tile but a workgroup's first
+// starts with an exposed round trip to memory.  Opt-in (spec ps=1): measured 169 against 160 us (fp64) and 100 against
+// 90 us (fp32) for the nine CCSD(T) terms -- two to six workgroups per CU in different phases already hide a tile's
+// start, and this kernel needs 40 more registers.  With an odd number of terms the two register sets (and, with two
+// operand regions, the regions) change roles from tile to tile: the tile body exists once per parity P, a term t of
+// the tile living in set (t + P) % 2.
+template <int NREGION, class G, class... Terms>
+__global__ __launch_bounds__(G::NT)
+void tc_group_persist_kernel(typename G::T* __restrict__ C, const TcGroupArgs<(int)sizeof...(Terms)> ga)
+{
+    typedef typename G::T T;
+    constexpr bool FULL = true;
+    constexpr int N = (int)sizeof...(Terms);
+    static_assert(N >= 2, "a group has two terms or more");
+    constexpr int NT = G::NT, VOL = G::TILE_VOL;
+    constexpr int MAXX = tc_max_of(PipeSlots<Terms, FULL>::X...), MAXY = tc_max_of(PipeSlots<Terms, FULL>::Y...);
+    T* const lds_c = (T*)tc_dynamic_lds;
+    T* const lds_ops = lds_c + VOL;
+    // (not const: every tile re-reads it through an empty asm, so that the per-lane offsets of all terms' slice
+    // elements, which do not change from tile to tile, are recomputed per tile instead of being kept in ~200
+    // registers across the tile loop, which is what the compiler otherwise does)
+    int tid = threadIdx.x;
+    constexpr int CV = (G::c_tile(0) % (16 / (int)sizeof(T)) == 0 && VOL % (NT * (16 / (int)sizeof(T))) == 0) ? 16 / (int)sizeof(T) : 1;
+    typedef T TCV __attribute__((ext_vector_type(CV), aligned(sizeof(T))));
+    typedef T TLV __attribute__((ext_vector_type(CV)));
+    constexpr int NEL = (VOL / CV + NT - 1) / NT;
+
+    // origin of tile b (tiles in the order of their origins in C's memory) and the address of its first element
+    auto decode = [&](unsigned b, int (&org)[G::NIDX]) -> T* {
+        int64_t baseC = 0;
+#pragma unroll
+        for (int i = 0; i < G::NIDX; i++) org[i] = 0;
+#pragma unroll
+        for (int j = 0; j < G::CR; j++) {
+            const int id = G::c_id(j);
+            const unsigned nb = (unsigned)ga.nblk[id];
+            org[id] = (int)(b % nb) * G::c_tile(j);
+            b /= nb;
+            baseC += (int64_t)org[id] * ga.sC[id];
+        }
+        return C + uniform64(baseC);
+    };
+    // element q of a tile in C's memory order: its offset from the tile's first element (the same for every tile)
+    auto c_offset = [&](unsigned q) -> unsigned {
+        unsigned off = 0;
+#pragma unroll
+        for (int j = 0; j < G::CR; j++) {
+            const unsigned t = (unsigned)G::c_tile(j);
+            off += (q % t) * (unsigned)ga.sC[G::c_id(j)];
+            q /= t;
+        }
+        return off;
+    };
+    auto c_read = [&](TLV (&v)[NEL], const T* Cb) {
+#pragma unroll
+        for (int i = 0; i < NEL; i++) {
+            const unsigned q = (unsigned)(tid + i * NT) * CV;
+            if (VOL % (NT * CV) == 0 || q < (unsigned)VOL) {
+                const TCV w = __builtin_nontemporal_load((const TCV*)(Cb + c_offset(q)));
+#pragma unroll
+                for (int e = 0; e < CV; e++) v[i][e] = w[e];
+            }
+        }
+    };
+    auto c_to_lds = [&](const TLV (&v)[NEL]) {
+#pragma unroll
+        for (int i = 0; i < NEL; i++) {
+            const unsigned q = (unsigned)(tid + i * NT) * CV;
+            if (VOL % (NT * CV) == 0 || q < (unsigned)VOL) *(TLV*)(lds_c + q) = v[i];
+        }
+    };
+    auto c_write = [&](T* Cb) {
+#pragma unroll
+        for (int i = 0; i < NEL; i++) {
+            const unsigned q = (unsigned)(tid + i * NT) * CV;
+            if (VOL % (NT * CV) == 0 || q < (unsigned)VOL) {
+                const TLV w = *(const TLV*)(lds_c + q);
+                TCV o;
+#pragma unroll
+                for (int e = 0; e < CV; e++) o[e] = w[e];
+                __builtin_nontemporal_store(o, (TCV*)(Cb + c_offset(q)));
+            }
+        }
+    };
+
+    typedef typename TermAt<0, Terms...>::type Term0;
+    typedef typename TermAt<(N > 1 ? 1 : 0), Terms...>::type Term1;
+    T px[2][MAXX], py[2][MAXY];
+    TLV v[NEL];
+    int org[G::NIDX], org_n[G::NIDX];
+    unsigned tile = blockIdx.x;
+    T* Cb = decode(tile, org);
+    T* Cb_n = Cb;
+    group_load<Term0, FULL, MAXX, MAXY>(px[0], py[0], ga, ga.term[0], org, tid);
+    if constexpr (N > 1) group_load<Term1, FULL, MAXX, MAXY>(px[1], py[1], ga, ga.term[1], org, tid);
+    c_read(v, Cb);
+    group_store<G, Term0, FULL, MAXX, MAXY>(px[0], py[0], lds_ops, ga, ga.term[0], org, tid);
+    c_to_lds(v);
+    __syncthreads();
+
+    // one tile.  HAS_NEXT is a template parameter, not a run-time test, so that a tile body holds no branch: the
+    // compiler's counts of outstanding loads stay exact at every wait (a branch around a load makes every later wait
+    // in the body a wait for everything).
+    auto body = [&](auto par, auto more) {
+        constexpr int P = decltype(par)::value;
+        constexpr bool HAS_NEXT = decltype(more)::value;
+        asm volatile("" : "+v"(tid));
+        static_for<N>([&](auto tt) {
+            constexpr int t = decltype(tt)::value;
+            constexpr int S = (t + P) & 1;                       // the set term t came from: free now
+            typedef typename TermAt<t, Terms...>::type Term;
+            typedef typename TermAt<(t + 1) % N, Terms...>::type Next;
+            typedef typename TermAt<(t + 2) % N, Terms...>::type Far;
+            if constexpr (t + 2 < N) group_load<Far, FULL, MAXX, MAXY>(px[S], py[S], ga, ga.term[t + 2], org, tid);
+            else if constexpr (HAS_NEXT) group_load<Far, FULL, MAXX, MAXY>(px[S], py[S], ga, ga.term[(t + 2) % N], org_n, tid);
+            if constexpr (t == N - 1 && HAS_NEXT) c_read(v, Cb_n);
+            group_contract<G, Term, FULL>(lds_c, lds_ops + (NREGION == 2 ? S : 0) * G::LDS_OPS, ga, ga.term[t], org, tid);
+            if constexpr (t + 1 < N || HAS_NEXT) {
+                if constexpr (NREGION == 1) __syncthreads();     // everybody is done reading the one region
+                group_store<G, Next, FULL, MAXX, MAXY>(px[S ^ 1], py[S ^ 1], lds_ops + (NREGION == 2 ? (S ^ 1) : 0) * G::LDS_OPS, ga,
+                                                       ga.term[(t + 1) % N], t + 1 < N ? org : org_n, tid);
+            }
+            __syncthreads();
+        });
+        c_write(Cb);
+        if constexpr (HAS_NEXT) {
+            // a lane overwrites exactly the elements it has just read; the barrier is for the other lanes' additions
+            c_to_lds(v);
+            __syncthreads();
+        }
+    };
+    const std::true_type yes;
+    const std::false_type no;
+    auto advance = [&](unsigned next) {
+        tile = next;
+        Cb = Cb_n;
+#pragma unroll
+        for (int i = 0; i < G::NIDX; i++) org[i] = org_n[i];
+    };
+    // two tiles per trip: with an odd number of terms the second one runs with the register sets exchanged
+    for (;;) {
+        unsigned next = tile + gridDim.x;
+        if (next >= ga.nblocks) { body(std::integral_constant<int, 0>(), no); break; }
+        Cb_n = decode(next, org_n);
+        body(std::integral_constant<int, 0>(), yes);
+        advance(next);
+        next = tile + gridDim.x;
+        if (next >= ga.nblocks) { body(std::integral_constant<int, N & 1>(), no); break; }
+        Cb_n = decode(next, org_n);
+        body(std::integral_constant<int, N & 1>(), yes);
+        advance(next);
+    }
+}
+
 // Host side.  inputs[] holds the 2 * NTERM input pointers in expression order (A of term 1, B of term 1,
 // A of term 2, ...); enabled[] (may be null: all) says which terms to apply; sizes[] as for tc_run.
 template <class G, class... Terms>
@@ -586,9 +742,33 @@ int tc_group_run(const int* sizes, void* C, const void* const* inputs, const int
             if (pipe_lds <= 160 * 1024) {
                 ok = ok && hipFuncSetAttribute((const void*)&tc_group_pipe_kernel<NREGION, false, G, Terms...>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pipe_lds) == hipSuccess;
                 ok = ok && hipFuncSetAttribute((const void*)&tc_group_pipe_kernel<NREGION, true, G, Terms...>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pipe_lds) == hipSuccess;
+                ok = ok && hipFuncSetAttribute((const void*)&tc_group_persist_kernel<NREGION, G, Terms...>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pipe_lds) == hipSuccess;
             }
             if (!ok) { (void)hipGetLastError(); return tc_fail(TC_ERR_LAUNCH, "the fused group kernel's LDS size was refused"); }
             configured[dev].store(true, std::memory_order_release);
+        }
+    }
+    if (pipe && full && G::PERSIST) {
+        // as many workgroups as the chip holds at once, each walking tiles blockIdx.x, + gridDim.x, ...
+        static std::atomic<int> slots[64];
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return tc_fail(TC_ERR_LAUNCH, "no current device for the fused group kernel");
+        int n_slots = slots[dev].load(std::memory_order_acquire);
+        if (n_slots == 0) {
+            int per_cu = 0, cus = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)&tc_group_persist_kernel<NREGION, G, Terms...>, G::NT, pipe_lds) != hipSuccess ||
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || per_cu < 1 || cus < 1) {
+                (void)hipGetLastError();
+                n_slots = -1;                          // no answer: the kernel with one workgroup per tile
+            } else {
+                n_slots = per_cu * cus;
+            }
+            slots[dev].store(n_slots, std::memory_order_release);
+        }
+        if (n_slots > 0) {
+            const unsigned g = (unsigned)std::min<int64_t>(grid, n_slots);
+            hipLaunchKernelGGL((tc_group_persist_kernel<NREGION, G, Terms...>), dim3(g), dim3(G::NT), pipe_lds, stream, (T*)C, ga);
+            return tc_check_launch("fused group kernel launch failed");
         }
     }
     if (pipe && full) hipLaunchKernelGGL((tc_group_pipe_kernel<NREGION, true, G, Terms...>), dim3((unsigned)grid), dim3(G::NT), pipe_lds, stream, (T*)C, ga);

@@ -158,7 +158,8 @@ bool plan_group(const std::vector<Contraction>& cs, DType t, const ArchGfx950& a
             else if (field.compare(0, 3, "kt=") == 0) g.k_room = std::max(4, std::min(64, atoi(field.c_str() + 3)));
             else if (field.compare(0, 3, "nw=") == 0) g.NW = std::max(1, std::min(8, atoi(field.c_str() + 3)));
             else if (field.compare(0, 3, "nr=") == 0) g.nregion = std::max(0, std::min(2, atoi(field.c_str() + 3)));
-            else { err = "group mapping spec: fields are ct=<tile>,... kt=<n> nw=<n> nr=<0|1|2>"; return false; }
+            else if (field.compare(0, 3, "ps=") == 0) g.persist = atoi(field.c_str() + 3) ? 1 : 0;
+            else { err = "group mapping spec: fields are ct=<tile>,... kt=<n> nw=<n> nr=<0|1|2> ps=<0|1>"; return false; }
         }
     }
     if (!ct_spec.empty()) {
@@ -208,7 +209,7 @@ std::string group_json(const GroupPlan& g)
     for (size_t j = 0; j < g.c_tile.size(); j++) o << (j ? ", " : "") << g.c_tile[j];
     o << "], \"threads\": " << 64 * g.NW << ", \"lds_bytes\": " << (g.vol + g.lds_ops) * esize(g.t) << ", \"spec\": \"ct=";
     for (size_t j = 0; j < g.c_tile.size(); j++) o << (j ? "," : "") << g.c_tile[j];
-    o << ";kt=" << g.k_room << ";nw=" << g.NW << ";nr=" << g.nregion << "\", \"terms\": [";
+    o << ";kt=" << g.k_room << ";nw=" << g.NW << ";nr=" << g.nregion << (g.persist ? ";ps=1" : "") << "\", \"terms\": [";
     for (size_t k = 0; k < g.terms.size(); k++)
         o << (k ? ", " : "") << "{\"text\": \"" << c_escape(g.terms[k].text) << "\", \"mapping\": " << mapping_json(g.terms[k], g.t, g.maps[k]) << "}";
     o << "]}";
@@ -233,7 +234,7 @@ std::string emit_group_source(const GroupPlan& g, const std::string& unique_name
     };
     o << "struct G {\n    typedef " << T << " T;\n";
     o << "    static constexpr int NIDX = " << c0.n_idx() << ", CR = " << c0.out_idx.size() << ", NTERM = " << N << ", NT = " << 64 * g.NW
-      << ", TILE_VOL = " << g.vol << ", LDS_OPS = " << g.lds_ops << ", NREGION = " << g.nregion << ";\n";
+      << ", TILE_VOL = " << g.vol << ", LDS_OPS = " << g.lds_ops << ", NREGION = " << g.nregion << ", PERSIST = " << g.persist << ";\n";
     table("c_id", c0.out_idx);
     table("c_tile", g.c_tile);
     o << "};\n";

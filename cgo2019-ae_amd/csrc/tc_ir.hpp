@@ -126,6 +126,7 @@ struct GroupPlan {
     std::vector<Mapping> maps;        // per term: roles and tiles derived from c_tile
     int NW = 4;                       // wavefronts per workgroup
     int k_room = 32;                  // contracted depth per K block
+    int persist = 0;                  // spec ps=1: for whole-tile calls, workgroups persistent over several tiles with the term pipeline running across tile boundaries (measured 6-10 % slower than one workgroup per tile: off)
     int nregion = 1;                  // operand regions in LDS of the pipelined kernel (spec nr=): 1 = more workgroups per CU, 2 = one barrier per term
     int vol = 0, lds_ops = 0;         // elements of the C tile; elements of the largest pair of operand slices
 };

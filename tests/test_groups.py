@@ -55,6 +55,8 @@ def test_group_tile_spec_and_rejections(tmp_path):
     assert rc == 0 and j["c_tile"] == [16, 2, 2, 4, 2, 2] and j["spec"] == "ct=16,2,2,4,2,2;kt=32;nw=4;nr=1"
     rc, j = plan_json(FUSED, spec="ct=16,4,4,2,2,2;kt=8;nw=8")                 # K depth per block, wavefronts per workgroup
     assert rc == 0 and j["threads"] == 512 and all(t["mapping"]["block_tile"][2] == 8 for t in j["terms"])
+    rc, j = plan_json(FUSED, spec="ct=16,4,4,2,2,2;kt=16;nw=4;nr=1;ps=1")     # persistent workgroups (opt-in)
+    assert rc == 0 and j["spec"].endswith(";ps=1")
     for nr in (0, 1, 2):                                               # operand regions of the pipelined kernel; 0 = the per-term kernel
         rc, j = plan_json(FUSED, spec="ct=16,4,4,2,2,2;kt=16;nw=4;nr=%d" % nr)
         assert rc == 0 and j["spec"].endswith(";nr=%d" % nr)
@@ -135,7 +137,8 @@ def group():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["fused_sd2_f64", "fused_sd1_f32", "var_fused_sd2_two_regions_f64", "var_fused_sd1_per_term_pass_f32"])
+@pytest.mark.parametrize("name", ["fused_sd2_f64", "fused_sd1_f32", "var_fused_sd2_two_regions_f64", "var_fused_sd2_persistent_f64",
+                                  "var_fused_sd1_per_term_pass_f32"])
 @pytest.mark.parametrize("sizes", [[5, 3, 7, 6, 2, 9, 4], [16, 4, 4, 2, 2, 2, 16], [17, 5, 6, 3, 4, 3, 19], [1, 1, 1, 1, 1, 1, 1],
                                    [32, 8, 4, 4, 4, 2, 24], [16, 16, 16, 16, 8, 8, 16]])
 def test_fused_group_matches_the_terms_applied_one_by_one(name, sizes, tools, oracle):
