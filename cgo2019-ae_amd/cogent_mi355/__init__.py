@@ -289,12 +289,12 @@ class Driver:
         arr = (ctypes.c_int * len(sizes))(*[int(s) for s in sizes])
         cb = (ctypes.c_void_p * len(c_ptrs))(*c_ptrs)
         each = (ctypes.c_float * iters)()
-        stats = (ctypes.c_float * 4)()
+        stats = (ctypes.c_float * 5)()
         rc = self.lib.cogent_driver_time(expr.path.encode(), arr, len(sizes), cb, len(c_ptrs), a_ptr, b_ptr,
                                          warmup, iters, variant, each, stats)
         if rc:
             raise CogentError("timing failed (%d): %s" % (rc, self.lib.cogent_driver_last_error().decode()))
-        return {"mean_ms": stats[0], "median_ms": stats[1], "min_ms": stats[2], "max_ms": stats[3], "each_ms": list(each)}
+        return {"mean_ms": stats[0], "median_ms": stats[1], "min_ms": stats[2], "max_ms": stats[3], "batch_mean_ms": stats[4], "each_ms": list(each)}
 
     def time_group(self, group, sizes, c_ptrs, input_ptrs, warmup, iters):
         self.lib.cogent_driver_time_group.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_int), ctypes.c_int,
@@ -306,12 +306,12 @@ class Driver:
         cb = (ctypes.c_void_p * len(c_ptrs))(*c_ptrs)
         ib = (ctypes.c_void_p * len(input_ptrs))(*input_ptrs)
         each = (ctypes.c_float * iters)()
-        stats = (ctypes.c_float * 4)()
+        stats = (ctypes.c_float * 5)()
         rc = self.lib.cogent_driver_time_group(group.path.encode(), arr, len(sizes), cb, len(c_ptrs), ib, len(input_ptrs),
                                                warmup, iters, each, stats)
         if rc:
             raise CogentError("timing failed (%d): %s" % (rc, self.lib.cogent_driver_last_error().decode()))
-        return {"mean_ms": stats[0], "median_ms": stats[1], "min_ms": stats[2], "max_ms": stats[3], "each_ms": list(each)}
+        return {"mean_ms": stats[0], "median_ms": stats[1], "min_ms": stats[2], "max_ms": stats[3], "batch_mean_ms": stats[4], "each_ms": list(each)}
 
     def time_rmw(self, buf_ptrs, nbytes, mode, warmup, iters):
         """Mean ms per launch of a bare read-modify-write of nbytes: mode 0 flat, 1 flat non-temporal, 2 / 3 in the tiles of the
