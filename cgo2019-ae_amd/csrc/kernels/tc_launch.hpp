@@ -46,9 +46,9 @@ inline int tc_check_launch(const char* what)
 
 enum TcVariant { TC_VARIANT_AUTO = 0, TC_VARIANT_PLAIN = 1, TC_VARIANT_TILED = 2, TC_VARIANT_VALU = 3 };
 // The VALU streaming kernel is never taken by TC_VARIANT_AUTO: measured at contracted extents 1, 2 and 3 (which do not
-// fill the 4-deep step of the fp64 / fp32 matrix instructions) it is 18 to 56 % SLOWER than the tiled kernel with the
-// slices zero-padded to one step (72^4 outer product 131 vs 111 us, 16^6 fp64 with 2 terms 70 vs 51 us, 16^6 fp32 with
-// 3 terms 51 vs 33 us): its per-element gathers of the inputs cost more issue slots than a padded matrix step.
+// fill the 4-deep step of the fp64 / fp32 matrix instructions) it is 45 to 85 % SLOWER than the tiled kernel with the
+// slices zero-padded to one step (72^4 outer product 131 vs 77 us, 16^6 fp64 with 2 terms 70 vs 48 us, 16^6 fp32 with
+// 3 terms 51 vs 28 us): its per-element gathers of the inputs cost more issue slots than a padded matrix step.
 
 // Which kernel the last call of this thread launched (0: none yet, or the call returned before a launch).
 enum TcKernelKind { TC_KERNEL_NONE = 0, TC_KERNEL_PLAIN = 1, TC_KERNEL_TILED = 2, TC_KERNEL_STREAM = 3, TC_KERNEL_VALU = 4 };
