@@ -380,6 +380,12 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     const double nX = m.x_is_a ? nA : nB, nY = m.x_is_a ? nB : nA;
     auto sector_eff = [&](const std::vector<int>& op) { return std::min(1.0, tile_of(op[0]) * s / 64.0); };
     m.t_hbm = (nX * s / sector_eff(xop) + nY * s / sector_eff(yop) + 2.0 * nC * s * c_passes * spread / c_hbm_eff) / (bw * occ_eff);
+    // a K loop in a memory-bound kernel: the variant without one requests its slices and its C tile together and has
+    // nothing else to wait for; with a loop a tile spends about a microsecond more in which it requests nothing from
+    // memory, and only the other workgroups of the CU keep the memory pipe busy meanwhile.  How MANY K blocks the loop
+    // has matters little (4-D shapes measured best with 18 blocks of 4).  The 6-D shapes with a 24-deep contracted
+    // index: one K block 107-129 us, blocks of 4 137-154 us.
+    if (nkb > 1 && m.STREAM == 0) m.t_hbm += (double)nblocks * 1.0e-6 / ((double)arch.n_cu * r);
     const double l1_bw = 64.0 * arch.n_cu * arch.clock_hz;
     const double t_l1 = 2.0 * nC * s * c_passes / (l1_bw * c_l1_eff);
 
@@ -414,7 +420,7 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     // (a block's wavefronts are dealt to the SIMDs starting at SIMD 0: 6 or 9 of them load the SIMDs unevenly;
     // measured: 6-wavefront blocks run 40% slower than 4-wavefront ones on the same tile volume)
     const double per_block = W >= arch.simd_per_cu ? ((double)W / arch.simd_per_cu) / std::ceil((double)W / arch.simd_per_cu) : 1.0;
-    const double simd_busy = std::min(waves_simd / std::ceil(waves_simd), per_block);
+    const double simd_busy = waves_simd / std::ceil(waves_simd);          // (uneven wavefront counts per workgroup: priced on the total below)
     const double n_mfma = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * (m.BXP / mi.MT) * (m.BYP / mi.MT);
     const double simd_hz = (double)arch.n_cu * arch.simd_per_cu * arch.clock_hz;
     // issue cycles next to the MFMAs, per wavefront and K block: loop, barrier and LDS operand reads
@@ -427,7 +433,16 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     // (the wavefronts of ONE workgroup meet at every barrier and so stall together: what counts is the number of
     // workgroups on the CU -- twelve wavefronts of one workgroup measured 64 % on config 3, where two workgroups
     // of four reached 77 % with a second K block requested ahead)
-    const double mfma_occ = std::min(0.95, (r >= 3 ? 0.92 : r == 2 ? 0.84 : 0.70) + (m.PD >= 2 ? 0.05 : 0.0));
+    // Both counts matter: one-wavefront workgroups, however many of them, leave every SIMD with a single wavefront that
+    // stages its slices alone (the DGEMM on 48x80 tiles of one wavefront measured 1.34 times its four-wavefront mapping).
+    // With a second K block in flight in registers the global loads are never exposed and a lone large workgroup keeps
+    // its matrix cores fed (4-D x 4-D shapes, 192x192 tiles on twelve wavefronts, 8-deep K blocks, pd=2: 78-84 % of
+    // peak).  Not with split K: there a workgroup ends with an atomic pass over its tile that only another workgroup
+    // of the CU can overlap (config 3, 144x192 tiles on twelve wavefronts, pd=2: 64 %); there it is worth five points.
+    const double by_groups = r >= 3 ? 0.92 : r == 2 ? 0.84 : 0.70;
+    const double by_waves = waves_simd >= 3.0 ? 0.92 : waves_simd >= 2.0 ? 0.84 : 0.68;
+    const double mfma_occ = (m.PD >= 2 && sk == 1) ? std::min(0.92, std::max(by_waves, by_groups + 0.05))
+                                                   : std::min(0.92, std::min(by_groups, by_waves) + (m.PD >= 2 ? 0.05 : 0.0));
     m.t_mfma = (n_mfma * mi.cycles / simd_hz / mfma_occ + t_overhead) / simd_busy;
 
     const double lds_reads = (double)nblocks * nkb * (m.BKP / mi.KSTEP) * W * (m.TX + m.TY) * 64.0 * s;
@@ -446,6 +461,17 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     // fabric as C, and the mappings measured best on the 6-D shapes were those with the least of it among near-equal
     // HBM terms)
     m.cost = (mx + 0.15 * (sum - mx) + (std::max(m.t_hbm, m.t_l2) >= mx ? 0.25 * std::min(m.t_l2, m.t_hbm) : 0.0)) * spill_penalty / std::max(m.tail_eff, 0.05) + 2.0e-6;
+    // workgroups whose wavefronts load the SIMDs unevenly are slow whatever binds (6 wavefronts: +40 % measured on an
+    // HBM-bound shape), and a tile that does not divide its representative extent sends every call at those extents to
+    // the predicated kernel variant (no vector accesses, edge tests in every access)
+    m.cost /= std::max(0.6, per_block);
+    {
+        bool ragged = false;
+        for (size_t i = 0; i < m.x_ids.size(); i++) ragged = ragged || (c.indices[m.x_ids[i]].rep_size % m.x_tiles[i]) != 0;
+        for (size_t i = 0; i < m.y_ids.size(); i++) ragged = ragged || (c.indices[m.y_ids[i]].rep_size % m.y_tiles[i]) != 0;
+        for (size_t i = 0; i < m.k_ids.size(); i++) ragged = ragged || (c.indices[m.k_ids[i]].rep_size % m.k_tiles[i]) != 0;
+        if (ragged) m.cost *= 1.10;
+    }
     // the streaming kernel must win clearly: on the 6-D shapes it measured level with the per-tile kernel for most
     // index orders and a third slower for some, which nothing above tells apart
     if (m.STREAM > 0) m.cost *= 1.05;
@@ -488,12 +514,26 @@ static int vector_sides(const Contraction& c, DType t, const Mapping& m)
 //   more (config 1: -5 %).
 static void measured_rules(const Contraction& c, DType t, Mapping& m)
 {
-    if (k_blocks(c, m) != 1) { m.VL = vector_sides(c, t, m); return; }
+    // C through LDS in memory order, with non-temporal accesses, when C's rows are not whole 128-byte lines (96-byte
+    // fp32 rows -5 %, 192-byte fp64 rows -3 to -5 % with one K block; the 3-D and 4-D shapes with 192-byte rows and a K
+    // loop 89 -> 70 us); not on whole-line rows (+12 %).  The cost model drops it where the tile exceeds 64 KB.
+    {
+        const long long row = (long long)m.x_tiles[0] * esize(t);
+        const bool fits = (long long)m.BX * m.BY * esize(t) <= 65536;
+        if (row % 128 != 0 && row % 16 == 0 && m.SK == 1 && fits) { m.clds_forced = 1; m.ntc_forced = 3; }
+    }
+    if (k_blocks(c, m) != 1) {
+        m.VL = vector_sides(c, t, m);
+        // a long K loop: a second K block in flight in registers (config 3 +12-17 %, the DGEMM and the 4-D x 4-D shapes
+        // +4-10 %), which pays where the register budget takes it: small slice shares per lane
+        const int W = m.WX * m.WY;
+        const int slots = (m.BK * m.BX + 64 * W - 1) / (64 * W) + (m.BK * m.BY + 64 * W - 1) / (64 * W);
+        if (k_blocks(c, m) / std::max(1, m.SK) >= 8 && slots <= 8) m.pd_forced = 2;
+        return;
+    }
     if (m.SK > 1) return;
     m.TORD = 1;
     m.VL = 1;
-    const long long row = (long long)m.x_tiles[0] * esize(t);
-    if (row % 128 != 0 && row % 16 == 0) m.clds_forced = 1;
 }
 
 // The streaming kernel for an enumerated mapping: depth 3 for three K blocks, else 2; C non-temporal; runs of the
@@ -504,7 +544,10 @@ static bool stream_variant(const Contraction& c, DType t, const ArchGfx950& arch
     const long long nkb = k_blocks(c, m);
     // three K blocks or more: with two, the kernel measured level with the per-tile kernel at best (config 4 with 16s,
     // some 6-D shapes) and a third to two thirds slower on others (config 4, config 5 #9), which nothing here tells apart
-    if (nkb < 3 || nkb > 64 || m.SK > 1) return false;
+    // (and no more: its design point is a handful of K blocks per tile; every win of this kernel that came out of these
+    // candidates had three.  On config 1 one tile shape with 16 K blocks measured 28 us, another, which the model
+    // priced lower, 52 us, and one with four 33 us against 30 us for the per-tile pick)
+    if (nkb != 3 || m.SK > 1) return false;
     if (t != DType::F64) return false;       // fp32: its one measured win had two K blocks; the six-index fp32 shape ran 1.7 to 2 times slower with it
     // every measured win of this kernel had eight or more wavefronts with at most three accumulator tiles each (its one
     // workgroup per CU is all that hides the memory latency; two wavefronts with 18 tiles each ran at half the
