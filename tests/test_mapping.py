@@ -223,3 +223,52 @@ def test_impossible_mappings_are_rejected(spec, tools):
     with pytest.raises(cogent_mi355.CogentError) as e:
         tools.plan(text, "DOUBLE", mapping_spec=spec)
     assert e.value.code == 3
+
+
+def _pick(tools, name, dtype="DOUBLE"):
+    return tools.plan(open(os.path.join(EXPR_DIR, name)).read(), dtype).info["mapping"]
+
+
+def test_first_picks_follow_the_measured_rules(tools):
+    """What the pass decides on its own (no spec, no tuned table), pinned where a measurement stands behind it."""
+    # config 2: whole aligned chunks of C (two full rows of d: 1152 bytes) and the streaming kernel at three K blocks
+    m = _pick(tools, "cfg2_f64.in")
+    assert m["x"] == [["d", 72], ["c", 2]] and m["k"] == [["e", 24]] and m["stream"] == [3, 3]
+    assert m["nontemporal_c"] == 3 and m["stream_interleaved_runs"] == 1 and m["stream_panel_overlap"] == 1
+    # the 6-D shapes keep a 24- or 16-deep contracted index in ONE K block; tiles then go out in C's memory order with
+    # 16-byte slice loads, and C passes through LDS where its rows are not whole 128-byte lines (192 bytes here)
+    m = _pick(tools, "tccg_31.in")
+    assert m["k"] == [["g", 24]] and m["model"]["k_steps"] == 1 and m["stream"][0] == 0
+    assert m["tile_order_c_memory"] == 1 and m["vector_slice_loads"] == 1 and m["c_through_lds"] == 1 and m["nontemporal_c"] == 3
+    m = _pick(tools, "cfg5_1_f64.in")                                  # 128-byte rows: no LDS copy of C
+    assert m["model"]["k_steps"] == 1 and m["tile_order_c_memory"] == 1 and m["c_through_lds"] == 0
+    # a K loop with 192-byte rows of C: C through LDS there too; no tile-order option on a K loop
+    m = _pick(tools, "tccg_03.in")
+    assert m["model"]["k_steps"] > 1 and m["c_through_lds"] == 1 and m["tile_order_c_memory"] == 0
+    # fp32 never gets the streaming kernel from the pass, nor does a shape with other than three K blocks
+    assert _pick(tools, "cfg4_16_f32.in", "FLOAT")["stream"][0] == 0
+    assert _pick(tools, "cfg1_f64.in")["stream"][0] == 0
+    # a long MFMA-bound K loop with small slice shares: a second K block in flight
+    m = _pick(tools, "tccg_20.in")
+    assert m["prefetch_depth"] == 2 and m["split_k"] == 1
+
+
+BENCH_FILES = [p for p in FILES if os.path.basename(p).startswith(("cfg", "tccg_", "ccsd_"))]
+
+
+@pytest.mark.parametrize("path", BENCH_FILES, ids=[os.path.basename(p) for p in BENCH_FILES])
+def test_first_pick_has_whole_tiles(path, tools):
+    """On the benchmark expressions whose extents are 16, 24, 32, 48, 72 or 256 every first pick divides the representative
+    extents, so that calls at those extents take the kernel variants without predicates (312 and 296 have no divisor that
+    is a multiple of the 16-wide matrix tile: there a ragged tile can be the better trade), and no workgroup has 6 or 9
+    wavefronts (which load the four SIMDs unevenly: +40 % measured)."""
+    text = open(path).read()
+    for dtype in (("FLOAT",) if path.endswith("_f32.in") else ("DOUBLE",)):          # the data type the object is shipped in
+        info = tools.plan(text, dtype).info
+        m = info["mapping"]
+        ext = dict(zip(info["out_idx"] + info["sum_idx"], info["rep_sizes"]))
+        if not set(ext.values()) <= {16, 24, 32, 48, 72, 256}:
+            return
+        for name, tile in m["x"] + m["y"] + m["k"]:
+            assert ext[name] % tile == 0, (name, tile, ext[name], m["spec"])
+        assert m["threads"] // 64 not in (6, 9), m["spec"]
