@@ -385,7 +385,15 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     // memory, and only the other workgroups of the CU keep the memory pipe busy meanwhile.  How MANY K blocks the loop
     // has matters little (4-D shapes measured best with 18 blocks of 4).  The 6-D shapes with a 24-deep contracted
     // index: one K block 107-129 us, blocks of 4 137-154 us.
-    if (nkb > 1 && m.STREAM == 0) m.t_hbm += (double)nblocks * 1.0e-6 / ((double)arch.n_cu * r);
+    // Likewise the first slices of a tile: until they are in LDS the tile computes nothing, and the wait grows with
+    // their size at about a CU's share of the memory bandwidth (one 55 KB slice pair per tile measured 1.3-1.4 times
+    // slower than 8-deep K blocks on the 5-D shapes; 41 KB against 7 KB 1.2 times on the 4-D shapes).
+    // (The variant without a K loop requests its slices together with its C tile and waits for both at once: no such
+    // term there, as long as the slices are no larger than the kernel was measured with, see the end of this function.)
+    if (m.STREAM == 0 && nkb > 1) {
+        const double fill = (double)m.BK * (m.BX + m.BY) * s / (arch.hbm_bytes_per_s / arch.n_cu);
+        m.t_hbm += (double)nblocks * (fill + 1.0e-6) / ((double)arch.n_cu * r);
+    }
     const double l1_bw = 64.0 * arch.n_cu * arch.clock_hz;
     const double t_l1 = 2.0 * nC * s * c_passes / (l1_bw * c_l1_eff);
 
@@ -461,6 +469,9 @@ void cost_model(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& 
     // fabric as C, and the mappings measured best on the 6-D shapes were those with the least of it among near-equal
     // HBM terms)
     m.cost = (mx + 0.15 * (sum - mx) + (std::max(m.t_hbm, m.t_l2) >= mx ? 0.25 * std::min(m.t_l2, m.t_hbm) : 0.0)) * spill_penalty / std::max(m.tail_eff, 0.05) + 2.0e-6;
+    // one K block with more than 32 KB of slices: measured 1.3-1.4 times slower than an 8-deep K loop (5-D shapes, 55 KB);
+    // 16 and 25 KB are where the one-block kernel wins (6-D shapes)
+    if (nkb == 1 && (double)m.BK * (m.BX + m.BY) * s > 32768.0) m.cost *= 1.3;
     // workgroups whose wavefronts load the SIMDs unevenly are slow whatever binds (6 wavefronts: +40 % measured on an
     // HBM-bound shape), and a tile that does not divide its representative extent sends every call at those extents to
     // the predicated kernel variant (no vector accesses, edge tests in every access)
@@ -566,13 +577,23 @@ static bool stream_variant(const Contraction& c, DType t, const ArchGfx950& arch
         }
         if (chunk % 128) return false;
     }
+    // the panel is worth keeping only if several tiles of the other side pass by it (with one, "resident" means an
+    // exposed panel load per tile: 167 against 126 us on the 4-D shapes whose second input is a 72x72 matrix)
+    {
+        long long streamed = 1;
+        const std::vector<int>& ids = m.SRES ? m.x_ids : m.y_ids;
+        const std::vector<int>& tiles = m.SRES ? m.x_tiles : m.y_tiles;
+        for (size_t i = 0; i < ids.size(); i++) streamed *= ceil_div(c.indices[ids[i]].rep_size, tiles[i]);
+        if (streamed < 4) return false;
+    }
     m.st_forced = nkb == 3 ? 3 : nkb % 2 == 0 ? 2 : nkb % 3 == 0 ? 3 : 0;
     if (m.st_forced == 0) return false;
     std::string err;
     if (!plan_stream(c, t, arch, m, err)) return false;
     m.ntc_forced = 3;
     m.SIL = 1;
-    const long long panel = (long long)esize(t) * nkb * (m.layx == 0 ? (long long)m.BKP * m.ldx : (long long)m.BXP * m.ldx);
+    const long long panel = (long long)esize(t) * nkb * (m.SRES ? (m.layy == 0 ? (long long)m.BKP * m.ldy : (long long)m.BYP * m.ldy)
+                                                                : (m.layx == 0 ? (long long)m.BKP * m.ldx : (long long)m.BXP * m.ldx));
     m.SOV = panel > 65536 ? 1 : 0;
     m.VL = vector_sides(c, t, m);
     return true;
@@ -691,8 +712,9 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
                         cost_model(c, t, arch, m);
                         out.push_back(m);
                         // the streaming kernel wherever it can run with this tile
-                        {
+                        for (int resident_y = 0; resident_y < 2; resident_y++) {
                             Mapping mv = m;
+                            mv.SRES = resident_y;          // either side's panel can be the resident one: the cost terms choose
                             if (stream_variant(c, t, arch, mv)) { cost_model(c, t, arch, mv); out.push_back(mv); }
                         }
                         // few output tiles and a long K loop: also try splitting K over 2, 4, 8 workgroups
