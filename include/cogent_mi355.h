@@ -81,7 +81,9 @@ const char* cogent_host_last_error(void);
 /* Fused group: `text` holds two or more expressions with the same output tensor, output index list,
  * summed indices and sizes (the reference's outer group, cogent/src/algs/bases/tc_gen_inputs.py:113-123;
  * the CCSD(T) terms of cogent/drivers/ccsd_t/code_main_sd2_1.c:573-606).  Plans one tile of the output
- * for the whole group (tile_spec NULL/"" = search, or "ct=<tile>,..." one per output index) and, when
+ * for the whole group (tile_spec NULL/"" = search, or "ct=<tile>,..." one per output index, optionally followed by
+ * ";kt=<K depth per block>;nw=<wavefronts per workgroup>;nr=<operand regions in LDS: 1, 2, or 0 for the kernel with one
+ * pass per term>;ps=<1: persistent workgroups>") and, when
  * out_path is given, writes ONE translation unit whose kernel keeps the output tile on chip across the
  * terms.  Returns 0; 1 parse error; 2 data type; 3 no admissible tile / expressions do not form a group;
  * 5 file.  cogent_group_last_json() describes the plan of the last successful call. */
