@@ -33,7 +33,7 @@ def plan_json(path, dtype="DOUBLE", spec=None):
 
 def test_group_plan_shares_one_tile_and_gives_each_term_its_own_roles():
     rc, j = plan_json(FUSED)
-    assert rc == 0 and j["group"] and j["n_terms"] == 9 and j["threads"] == 256
+    assert rc == 0 and j["group"] and j["n_terms"] == 9 and j["threads"] == 512           # 4096-element tile: eight wavefronts
     assert j["out_idx"] == ["h3", "h2", "h1", "p6", "p5", "p4"] and j["sum_idx"] == ["p7"]
     tile = dict(zip(j["out_idx"], j["c_tile"]))
     vol = int(np.prod(j["c_tile"]))
@@ -45,7 +45,7 @@ def test_group_plan_shares_one_tile_and_gives_each_term_its_own_roles():
         assert got == tile
         assert m["x"][0][0] == "h3"                         # the output's fastest index leads the X side
         assert m["block_tile"][0] * m["block_tile"][1] == vol
-        assert m["threads"] == 256 and m["split_k"] == 1
+        assert m["threads"] == 512 and m["split_k"] == 1
     # the nine terms do not agree on which input is the X side, nor on the split of the externals
     assert len({tuple(n for n, _ in t["mapping"]["x"]) for t in j["terms"]}) > 1
 
