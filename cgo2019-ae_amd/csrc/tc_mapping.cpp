@@ -740,12 +740,43 @@ std::vector<Mapping> enumerate_mappings(const Contraction& c, DType t, const Arc
     return out;
 }
 
+// The pass's own pick with a long K loop and one K block requested ahead: the same tile with 8-deep K blocks and two of
+// them in flight, when the smaller slices bring the staged elements per lane within the budget of that option.  The
+// cost terms prefer deep K blocks (fewer barriers and loop trips) and do not see that a single block's matrix steps
+// are too short to cover the load latency.  Measured, same tile both ways (fp64): 3-D x 2-D shapes with K = 296,
+// 16- or 24-deep against 8-deep with two ahead 388 -> 336 us and 362 -> 340 us; the 2-D output with K = 92,000,
+// 32-deep 440 -> 8-deep 360 us; config 3, 24-deep 407 -> 398 us.
+static void deepen_prefetch(const Contraction& c, DType t, const ArchGfx950& arch, Mapping& pick)
+{
+    if (t != DType::F64 || pick.STREAM != 0 || pick.PD >= 2 || pick.k_ids.empty()) return;
+    if (pick.BK <= 8 || pick.k_tiles[0] < 8 || c.indices[pick.k_ids[0]].rep_size % 8 != 0) return;
+    // only where the matrix cores set the pace (a memory-bound 4-D shape lost 6 % with it) ...
+    if (pick.t_mfma < std::max(pick.t_hbm, pick.t_l2)) return;
+    Mapping m = pick;
+    m.k_tiles[0] = 8;
+    // ... and no input may lose the tile along its fastest index (4-D x 4-D and 3-D x 3-D shapes whose second
+    // contracted index is an input's fastest one: 1.1 to 2.6 times slower with that tile at 1)
+    for (size_t i = 1; i < m.k_tiles.size(); i++) {
+        if (m.k_tiles[i] > 1 && (m.k_ids[i] == c.a_idx[0] || m.k_ids[i] == c.b_idx[0])) return;
+        m.k_tiles[i] = 1;
+    }
+    finish_geometry(c, t, m);
+    std::string err;
+    if (!check_mapping(c, t, arch, m, err)) return;
+    m.pd_forced = -1;
+    measured_rules(c, t, m);
+    if (m.pd_forced != 2) return;               // still too many staged elements per lane, or too few K blocks
+    cost_model(c, t, arch, m);
+    if (m.PD != 2) return;
+    pick = m;
+}
+
 bool select_mapping(const Contraction& c, DType t, const ArchGfx950& arch, int rank, Mapping& out, std::string& err)
 {
     std::vector<Mapping> all = enumerate_mappings(c, t, arch);
     if (all.empty()) { err = "no admissible mapping for this expression"; return false; }
     if (rank >= 0 && rank < (int)all.size()) out = all[rank];   // manual pick, configurations.py:285-289
-    else out = all[0];
+    else { out = all[0]; deepen_prefetch(c, t, arch, out); }
     return true;
 }
 

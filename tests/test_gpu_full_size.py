@@ -115,3 +115,63 @@ def test_contracted_extents_that_do_not_fill_a_matrix_step(name, k, tools, oracl
     if k == 1:
         # a single term per element: one product and one sum, the oracle's two roundings or the fused one
         assert helpers.rel_error(got, want) <= (3e-16 if ex.dtype == "f64" else 2e-7)
+
+
+def _factor_tensor(torch, idx_list, ext, tdtype, skip=()):
+    """Column-major tensor over idx_list whose value is the product of (i mod 3) + 1 over its indices not in `skip`
+    (small integers: every product and sum below is exact in fp64 and fp32)."""
+    shape = [ext[i] for i in reversed(idx_list)]                 # torch is row-major: slowest index first
+    t = torch.ones(shape, dtype=tdtype, device="cuda")
+    for pos, i in enumerate(reversed(idx_list)):
+        if i in skip:
+            continue
+        view = [1] * len(shape)
+        view[pos] = ext[i]
+        t *= ((torch.arange(ext[i], device="cuda") % 3) + 1).to(tdtype).view(view)
+    return t.reshape(-1)
+
+
+# name, extents (output indices then contracted ones), the kernel expected to run
+BEYOND_4_GIB = [
+    ("tccg_12_f64", [24576, 24608, 16], "tiled"),                      # 2-D output, K loop: 4.84 GB
+    ("cfg5_1_f64", [32, 32, 32, 32, 32, 18, 4], "tiled"),              # 6-D output, one K block, ragged: 4.83 GB
+    ("cfg2_f64", [72, 72, 72, 1504, 72], "stream"),                   # the streaming kernel: 4.49 GB
+    ("cfg4_16_f32", [16, 16, 16, 16, 16, 1040, 16], None),                      # fp32: 4.36 GB
+]
+
+
+@pytest.mark.parametrize("name,sizes,kernel", BEYOND_4_GIB, ids=[c[0] for c in BEYOND_4_GIB])
+def test_output_beyond_4_gib(name, sizes, kernel, tools):
+    """Outputs of more than 2^32 bytes: tile origins are 64-bit, offsets inside a tile 32-bit.  Inputs are products of
+    per-index factors (i mod 3) + 1 over their external indices, so C[...] = (product of the contracted extents) x the
+    product of the factors of ALL its indices: an origin that wrapped, a tile done twice or left out, or an index taken
+    for another shows as a wrong integer somewhere.  Checked over every element, on the device, exactly."""
+    import torch
+    import cogent_mi355 as pkg
+    ex = pkg.Expression(name)
+    expr = helpers.parse_expression(pkg.expression_text(name))
+    tdtype = torch.float64 if ex.dtype == "f64" else torch.float32
+    ext = dict(zip(expr["all_idx"], sizes))
+    nC, nA, nB = helpers.tensor_sizes(expr, sizes)
+    assert nC * (8 if ex.dtype == "f64" else 4) > 2**32 and nC < 2**31
+    print("[gpu] beyond 4 GiB %s %s" % (name, sizes), flush=True)
+    a = _factor_tensor(torch, expr["a_idx"], ext, tdtype, skip=expr["sum_idx"])
+    b = _factor_tensor(torch, expr["b_idx"], ext, tdtype, skip=expr["sum_idx"])
+    assert a.numel() == nA and b.numel() == nB
+    c = torch.zeros(nC, dtype=tdtype, device="cuda")
+    assert ex.entry(sizes, c.data_ptr(), a.data_ptr(), b.data_ptr()) == 0, ex.last_error()
+    torch.cuda.synchronize()
+    if kernel:
+        assert ex.last_kernel() == kernel, ex.last_kernel()
+    # divide the factors out again, in place (exact: every value is a small integer multiple of them)
+    shape = [ext[i] for i in reversed(expr["out_idx"])]
+    cv = c.view(shape)
+    for pos, i in enumerate(reversed(expr["out_idx"])):
+        view = [1] * len(shape)
+        view[pos] = ext[i]
+        cv /= ((torch.arange(ext[i], device="cuda") % 3) + 1).to(tdtype).view(view)
+    ksize = float(np.prod([ext[i] for i in expr["sum_idx"]]))
+    sign = -1.0 if expr["op"] == "-=" else 1.0
+    assert bool((c == sign * ksize).all())
+    del c, cv, a, b
+    torch.cuda.empty_cache()

@@ -251,6 +251,21 @@ def test_first_picks_follow_the_measured_rules(tools):
     # a long MFMA-bound K loop with small slice shares: a second K block in flight
     m = _pick(tools, "tccg_20.in")
     assert m["prefetch_depth"] == 2 and m["split_k"] == 1
+    # ... and where the pick has deep K blocks with one ahead, the same tile is emitted with 8-deep blocks and two ahead
+    # (the ranked list itself is untouched: rank 0 asked for by number is the 24-deep mapping)
+    m = _pick(tools, "cfg3_f64.in")
+    assert m["k"] == [["e", 8], ["f", 1]] and m["prefetch_depth"] == 2 and m["split_k"] == 2
+    ranked0 = tools.plan(open(os.path.join(EXPR_DIR, "cfg3_f64.in")).read(), "DOUBLE", config_rank=0).info["mapping"]
+    assert ranked0["k"] == [["e", 24], ["f", 1]] and ranked0["prefetch_depth"] == 1
+    assert (ranked0["x"], ranked0["y"], ranked0["waves"]) == (m["x"], m["y"], m["waves"])
+    m = _pick(tools, "tccg_16.in")
+    assert m["k"] == [["d", 8]] and m["prefetch_depth"] == 2
+    # not where a second contracted index is an input's fastest one (its tile would drop to 1) ...
+    m = _pick(tools, "tccg_30.in")
+    assert m["prefetch_depth"] == 1 and dict(map(tuple, m["k"]))["e"] > 1
+    # ... nor on a memory-bound shape
+    m = _pick(tools, "tccg_05.in")
+    assert m["k"] == [["e", 12]] and m["prefetch_depth"] == 1
 
 
 BENCH_FILES = [p for p in FILES if os.path.basename(p).startswith(("cfg", "tccg_", "ccsd_"))]
