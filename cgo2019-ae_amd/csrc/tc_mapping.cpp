@@ -544,7 +544,11 @@ static void measured_rules(const Contraction& c, DType t, Mapping& m)
     }
     if (m.SK > 1) return;
     m.TORD = 1;
-    m.VL = 1;
+    // 16-byte slice loads by the same 64-byte rule as with a K loop.  Runs of 128 bytes on both sides: -1 to -2 % on the
+    // 6-D shapes at extent 16.  A side with 32-byte runs loaded that way: +6 % on the 6-D shapes at extents 24/16.  The
+    // long side alone there: -5 % on the picks with four wavefronts in a row and on config 4 at 24s, +3 % on the picks
+    // with two by two (no vector loads at all would suit those, and cost the others 2 to 7 %).
+    m.VL = vector_sides(c, t, m);
 }
 
 // The streaming kernel for an enumerated mapping: depth 3 for three K blocks, else 2; C non-temporal; runs of the

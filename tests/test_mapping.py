@@ -125,9 +125,10 @@ def test_kernel_options_in_a_spec(tools):
     auto = tools.plan(text4, "FLOAT", mapping_spec="x=0:16,2:16,4:1;y=1:16,3:2,5:1;k=6:16;w=4x1;t=4x2;mi=1").info["mapping"]
     assert auto["swapped_roles"] == 1 and auto["nontemporal_c"] == 0           # 64-byte rows: no whole lines per access
     # the pass's own pick for this shape (one K block, rows that are not whole lines): C through LDS in memory order,
-    # whose tile is made of whole lines, tiles in C's memory order, 16-byte slice loads
+    # whose tile is made of whole lines, tiles in C's memory order, 16-byte slice loads on the side whose runs reach 64
+    # bytes (the Y input's 16 floats; the X input's runs are 8 floats here)
     pick = tools.plan(text4, "FLOAT").info["mapping"]
-    assert pick["c_through_lds"] == 1 and pick["tile_order_c_memory"] == 1 and pick["vector_slice_loads"] == 1 and pick["stream"][0] == 0
+    assert pick["c_through_lds"] == 1 and pick["tile_order_c_memory"] == 1 and pick["vector_slice_loads"] == 3 and pick["stream"][0] == 0
     off = tools.plan(text4, "FLOAT", mapping_spec=auto["spec"] + ";sw=0").info["mapping"]
     assert off["swapped_roles"] == 0
     # fp64 rows of 16 elements are whole aligned lines: non-temporal loads and stores
@@ -239,9 +240,10 @@ def test_first_picks_follow_the_measured_rules(tools):
     # 16-byte slice loads, and C passes through LDS where its rows are not whole 128-byte lines (192 bytes here)
     m = _pick(tools, "tccg_31.in")
     assert m["k"] == [["g", 24]] and m["model"]["k_steps"] == 1 and m["stream"][0] == 0
-    assert m["tile_order_c_memory"] == 1 and m["vector_slice_loads"] == 1 and m["c_through_lds"] == 1 and m["nontemporal_c"] == 3
-    m = _pick(tools, "cfg5_1_f64.in")                                  # 128-byte rows: no LDS copy of C
-    assert m["model"]["k_steps"] == 1 and m["tile_order_c_memory"] == 1 and m["c_through_lds"] == 0
+    assert m["tile_order_c_memory"] == 1 and m["c_through_lds"] == 1 and m["nontemporal_c"] == 3
+    assert m["vector_slice_loads"] == 3               # 16-byte loads for the input with 192-byte runs, not for the one with 32-byte runs
+    m = _pick(tools, "cfg5_1_f64.in")                                  # 128-byte rows: no LDS copy of C; 128-byte runs in both inputs
+    assert m["model"]["k_steps"] == 1 and m["tile_order_c_memory"] == 1 and m["c_through_lds"] == 0 and m["vector_slice_loads"] == 1
     # a K loop with 192-byte rows of C: C through LDS there too; no tile-order option on a K loop
     m = _pick(tools, "tccg_03.in")
     assert m["model"]["k_steps"] > 1 and m["c_through_lds"] == 1 and m["tile_order_c_memory"] == 0

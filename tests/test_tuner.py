@@ -133,6 +133,9 @@ def test_small_tile_shapes():
     assert specs == ["x=a:24,d:4,f:1;y=b:16,c:2,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1",
                      "x=a:24,d:4,f:1;y=b:16,c:2,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1;nt=3",
                      "x=a:24,d:4,f:1;y=b:8,c:4,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1",
-                     "x=a:24,d:4,f:1;y=b:8,c:4,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1;nt=3"]
+                     "x=a:24,d:4,f:1;y=b:8,c:4,e:1;k=g:24;w=2x2;t=3x1;mi=0;cl=1;nt=3",
+                     # ... and the 192x32 tile on four wavefronts side by side
+                     "x=a:24,d:8,f:1;y=b:8,c:4,e:1;k=g:24;w=4x1;t=3x2;mi=0;cl=1;to=1;vl=1",
+                     "x=a:24,d:8,f:1;y=b:8,c:4,e:1;k=g:24;w=4x1;t=3x2;mi=0;cl=1;to=1;vl=1;nt=3"]
     assert tuner.small_tile_shapes({"x": [["a", 64], ["b", 1]], "y": [["c", 8], ["d", 8]], "k": [["e", 8]]},
                                    dict(zip("abcde", [72] * 5)), "DOUBLE") == []
