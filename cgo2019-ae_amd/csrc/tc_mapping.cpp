@@ -518,11 +518,11 @@ static int vector_sides(const Contraction& c, DType t, const Mapping& m)
 // Options that the cost terms do not separate, set the way they measured best on the part.  (A mapping spec sets
 // them itself; these rules only act on the mappings the pass enumerates.)
 //   One K block (the many-index shapes whose cost is the traffic of C): tiles handed out in the order of their
-//   origins in C's memory, -7 to -12 % on the 6-D shapes of the benchmark set; 16-byte slice loads where a tile
-//   allows, -1 to -2 %; C through LDS when C's rows are not whole 128-byte lines (96-byte fp32 rows, 192-byte
-//   fp64 rows: -5 % and -3 to -5 %), not otherwise (+12 % on 128-byte rows).
-//   Several K blocks: 16-byte slice loads for the inputs whose tile along their fastest index spans half a line or
-//   more (config 1: -5 %).
+//   origins in C's memory, -7 to -12 % on the 6-D shapes of the benchmark set; C through LDS when C's rows are not
+//   whole 128-byte lines (96-byte fp32 rows, 192-byte fp64 rows: -5 % and -3 to -5 %), not otherwise (+12 % on
+//   128-byte rows).
+//   With or without a K loop: 16-byte slice loads for the inputs whose tile along their fastest index spans half a
+//   line or more (config 1: -5 %; figures for one K block at the rule itself).
 static void measured_rules(const Contraction& c, DType t, Mapping& m)
 {
     // C through LDS in memory order, with non-temporal accesses, when C's rows are not whole 128-byte lines (96-byte
