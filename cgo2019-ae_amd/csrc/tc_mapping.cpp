@@ -548,7 +548,20 @@ static void measured_rules(const Contraction& c, DType t, Mapping& m)
     // 6-D shapes at extent 16.  A side with 32-byte runs loaded that way: +6 % on the 6-D shapes at extents 24/16.  The
     // long side alone there: -5 % on the picks with four wavefronts in a row and on config 4 at 24s, +3 % on the picks
     // with two by two (no vector loads at all would suit those, and cost the others 2 to 7 %).
-    m.VL = vector_sides(c, t, m);
+    // ... and only where the vectors fill the workgroup's lanes well enough to save instructions: a side is loaded in
+    // ceil(elements / lanes) rounds of 8-byte loads or ceil(vectors / lanes) rounds of 16-byte ones, and a 16-byte
+    // round costs about one and a half 8-byte rounds (a 32x24 fp64 slice on 256 lanes: 3 rounds against 2, the second
+    // half empty, measured +3 %; 48x24: 5 against 3, -2 to -5 %; 128x16: 8 against 4, -1 to -2 %)
+    {
+        const int side = vector_sides(c, t, m);
+        const int lanes = 64 * m.WX * m.WY, v = 16 / esize(t);
+        auto pays = [&](int ext_tile) {
+            const int elems = m.BK * ext_tile;
+            return 3 * ceil_div(ceil_div(elems, v), lanes) < 2 * ceil_div(elems, lanes);
+        };
+        const bool vx = (side == 1 || side == 2) && pays(m.BX), vy = (side == 1 || side == 3) && pays(m.BY);
+        m.VL = vx && vy ? 1 : vx ? 2 : vy ? 3 : 0;
+    }
 }
 
 // The streaming kernel for an enumerated mapping: depth 3 for three K blocks, else 2; C non-temporal; runs of the

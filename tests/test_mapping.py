@@ -241,7 +241,10 @@ def test_first_picks_follow_the_measured_rules(tools):
     m = _pick(tools, "tccg_31.in")
     assert m["k"] == [["g", 24]] and m["model"]["k_steps"] == 1 and m["stream"][0] == 0
     assert m["tile_order_c_memory"] == 1 and m["c_through_lds"] == 1 and m["nontemporal_c"] == 3
-    assert m["vector_slice_loads"] == 3               # 16-byte loads for the input with 192-byte runs, not for the one with 32-byte runs
+    # no 16-byte slice loads: one input has 32-byte runs, the other's 32x24 slice would fill two rounds of 256 lanes half
+    assert m["vector_slice_loads"] == 0
+    m = _pick(tools, "tccg_32.in")                    # its 48x24 slice with 192-byte runs: three 16-byte rounds against five
+    assert m["vector_slice_loads"] == 2
     m = _pick(tools, "cfg5_1_f64.in")                                  # 128-byte rows: no LDS copy of C; 128-byte runs in both inputs
     assert m["model"]["k_steps"] == 1 and m["tile_order_c_memory"] == 1 and m["c_through_lds"] == 0 and m["vector_slice_loads"] == 1
     # a K loop with 192-byte rows of C: C through LDS there too; no tile-order option on a K loop
