@@ -233,6 +233,10 @@ def prepare(name, top_k=6, extra_specs=(), jobs=8, out_root=TUNING):
     # (config 4 at 24s: 276 -> 258 us; the 16^6 fp64 shapes -3 % to +5 %)
     specs += [sp + ";to=1" for sp in specs if "st=" not in sp and "sk=" not in sp and "to=" not in sp
               and cands and cands[0]["model"]["k_steps"] * max(1, cands[0]["split_k"]) == 1]
+    # C through LDS: also with the first slices requested before the C tile is staged (their round trip to L2 then
+    # overlaps the tile's to HBM, for the price of registers held through the staging: -11 % on a 96x64 fp32 tile,
+    # +3 to +7 % on three others)
+    specs += [sp + ";es=1" for sp in specs if "cl=1" in sp and "es=" not in sp]
     # split K: also with the K shares outermost over the grid, so that the tiles of one share meet in one L2
     specs += [sp + ";so=1" for sp in specs if "sk=" in sp and "so=" not in sp and "pd=" not in sp]
     if entry.get("map") and entry["map"] not in specs:

@@ -473,6 +473,19 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
         }
         return off;
     };
+    // Slices of the first K block.  Cfg::ESL with the C tile through LDS: they are requested BEFORE the tile is staged
+    // (two barriers that no load may cross stand between the staging and the K loop: requested behind them, the
+    // slices' round trip to L2 follows the tile's round trip to HBM instead of overlapping it).  The slices then sit
+    // in registers through the staging, which can cost a resident wavefront: measured -11 % on a 96x64 fp32 tile of a
+    // 6-D shape, +3 to +7 % on three other tiles, hence an option.  CL implies no split K, so the first block is at
+    // the origin of both slices.
+    constexpr int PD = ONE_KB ? 1 : Cfg::PD;
+    T rx[PD][SLOTS_X], ry[PD][SLOTS_Y];
+    constexpr bool EARLY = CL && (Cfg::ESL != 0);
+    if (EARLY) {
+        slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx[0], Xb, d, rem, tid);
+        slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry[0], Yb, d, rem, tid);
+    }
     if (CL) {
         TV cv[NVEC];
 #pragma unroll
@@ -556,8 +569,6 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
     // each depth in registers of its own (stage kb % PD, a compile-time index in every copy of the
     // trip below).  One trip of MFMA work is a fraction of a microsecond; a slice gathered through a
     // busy L2 takes several times that, so one stage of look-ahead leaves the loop waiting on loads.
-    constexpr int PD = ONE_KB ? 1 : Cfg::PD;
-    T rx[PD][SLOTS_X], ry[PD][SLOTS_Y];
     int64_t kxh = kx0, kyh = ky0;                  // slice origin of the newest K block requested
     int head = 0;                                  // ... and its number within this workgroup's share
     // Move the head one K block on (first composite K index fastest) -- unless it is at the last one:
@@ -580,8 +591,10 @@ void tc_mfma_kernel(typename Cfg::T* __restrict__ C, const typename Cfg::T* __re
             }
         }
     };
-    slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx[0], Xb + uniform64(kxh), d, rem, tid);
-    slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry[0], Yb + uniform64(kyh), d, rem, tid);
+    if (!EARLY) {
+        slice_load<Cfg, OX, EXT_FULL, INT_FULL>(rx[0], Xb + uniform64(kxh), d, rem, tid);
+        slice_load<Cfg, OY, EXT_FULL, INT_FULL>(ry[0], Yb + uniform64(kyh), d, rem, tid);
+    }
 #pragma unroll
     for (int s = 1; s < PD; s++) {
         advance_head();

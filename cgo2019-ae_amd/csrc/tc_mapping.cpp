@@ -75,6 +75,7 @@ std::string Mapping::spec() const
     if (SRES) o << ";sy=1";
     if (SOV) o << ";ov=1";
     if (TORD) o << ";to=1";
+    if (ESL) o << ";es=1";
     if (SIL) o << ";il=1";
     if (SCD > 1) o << ";cd=" << SCD;
     if (DBUF) o << ";db=1";
@@ -532,6 +533,10 @@ static void measured_rules(const Contraction& c, DType t, Mapping& m)
         const long long row = (long long)m.x_tiles[0] * esize(t);
         const bool fits = (long long)m.BX * m.BY * esize(t) <= 65536;
         if (row % 128 != 0 && row % 16 == 0 && m.SK == 1 && fits) { m.clds_forced = 1; m.ntc_forced = 3; }
+        // ... in fp32 with the first slices requested before the tile is staged (nine 6-D shapes at extents 24/16
+        // -5 to -11 %, config 4 at 24s -3 %; fp64 shapes 0 to +7 %: the slices held in registers through the staging
+        // cost a resident wavefront there)
+        if (m.clds_forced == 1 && t == DType::F32) m.ESL = 1;
     }
     if (k_blocks(c, m) != 1) {
         m.VL = vector_sides(c, t, m);
@@ -890,6 +895,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "sy") m.SRES = atoi(val.c_str()) ? 1 : 0;
         else if (key == "ov") m.SOV = atoi(val.c_str()) ? 1 : 0;
         else if (key == "to") m.TORD = atoi(val.c_str()) ? 1 : 0;
+        else if (key == "es") m.ESL = atoi(val.c_str()) ? 1 : 0;
         else if (key == "il") m.SIL = atoi(val.c_str()) ? 1 : 0;
         else if (key == "cd") m.SCD = std::max(1, std::min(2, atoi(val.c_str())));
         else if (key == "rx") m.RPX = atoi(val.c_str()) ? 1 : 0;
@@ -940,7 +946,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"split_k_outermost\": " << m.SKO << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"stream_resident\": \"" << (m.SRES ? "y" : "x") << "\", \"stream_panel_overlap\": " << m.SOV << ", \"stream_c_distance\": " << m.SCD << ", \"stream_interleaved_runs\": " << m.SIL << ", \"tile_order_c_memory\": " << m.TORD << ", \"dynamic_lds_stages\": " << m.DBUF << ", \"vector_slice_loads\": " << m.VL << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"split_k_outermost\": " << m.SKO << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"stream_resident\": \"" << (m.SRES ? "y" : "x") << "\", \"stream_panel_overlap\": " << m.SOV << ", \"stream_c_distance\": " << m.SCD << ", \"stream_interleaved_runs\": " << m.SIL << ", \"tile_order_c_memory\": " << m.TORD << ", \"early_slices\": " << m.ESL << ", \"dynamic_lds_stages\": " << m.DBUF << ", \"vector_slice_loads\": " << m.VL << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

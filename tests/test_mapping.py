@@ -90,6 +90,13 @@ def test_kernel_options_in_a_spec(tools):
     assert "pd=3" in m["spec"] and "nt=2" in m["spec"]
     again = tools.plan(text, "DOUBLE", mapping_spec=m["spec"]).info["mapping"]
     assert again == m
+    # es=1: the first slices requested before the C tile is staged through LDS (an option of cl=1 mappings; off by default)
+    small = "x=d:24,c:4;y=b:8,a:4;k=e:8;w=2x2;t=3x1"                      # a 24 KB tile: cl=1 needs at most 64 KB
+    m = tools.plan(text, "DOUBLE", mapping_spec=small + ";cl=1").info["mapping"]
+    assert m["c_through_lds"] == 1 and m["early_slices"] == 0 and "es=" not in m["spec"]
+    m = tools.plan(text, "DOUBLE", mapping_spec=small + ";cl=1;es=1").info["mapping"]
+    assert m["early_slices"] == 1 and m["spec"].endswith(";es=1")
+    assert tools.plan(text, "DOUBLE", mapping_spec=m["spec"]).info["mapping"] == m
     # rx=/ry=: an input copied into tile order first; its slices then go to LDS K-major whatever its own order
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:24,a:2;k=e:12;w=3x1;t=3x3;rx=1;ry=1").info["mapping"]
     assert m["repack"] == [1, 1] and m["lds_layout"] == [0, 0] and "rx=1" in m["spec"] and "ry=1" in m["spec"]
