@@ -15,6 +15,7 @@ hipcc cross-compiles for gfx950 without a GPU, so this runs on a CPU-only machin
 import concurrent.futures
 import json
 import os
+import re
 import subprocess
 import sys
 
@@ -131,7 +132,8 @@ def emit_and_compile(entry):
     """Emits and compiles one expression.  The compiler's resource report of every kernel in the object goes to
     lib/<name>.resources.json ("hot" names the instantiation that runs at the entry's benchmark extents).  If THAT
     kernel spills registers to scratch memory the build fails (such kernels ran 15 to 20 times slower when they were
-    measured) unless the entry says "allow_scratch"; spills in the variants for other extents are recorded only."""
+    measured) unless the entry says "allow_scratch"; spills in the variants for other extents are recorded, and where
+    they are the one-K-block kernels for ragged tiles the object is emitted again so that it no longer uses them."""
     name = entry["name"]
     hip = os.path.join(GEN, name + ".hip")
     cmd = [os.path.join(BIN, "cogent_gen"), name, os.path.join(EXPR, entry["file"]),
@@ -142,10 +144,29 @@ def emit_and_compile(entry):
     plan = json.loads(run(cmd))
     remarks = run(["hipcc"] + HIPCC_FLAGS + [RESOURCE_FLAG, "-o", os.path.join(LIB, name + ".so"), hip])
     res = kernel_resources(remarks)
-    spilling = sorted(k for k, v in res.items() if v.get("scratch_bytes", 0) > 0 and k.startswith(("tc_mfma", "tc_stream", "tc_group")))
+    is_spilling = lambda r: sorted(k for k, v in r.items() if v.get("scratch_bytes", 0) > 0 and k.startswith(("tc_mfma", "tc_stream", "tc_group")))
+    spilling = is_spilling(res)
+    # A one-K-block kernel for calls with ragged tiles (tc_mfma_kernel<E,I,1,*> other than E = I = 1) that spills: emit
+    # the object again with ok=0, which sends those calls through the K-loop kernels (a loop of one trip) instead.  Only
+    # for mappings without split K (the generator refuses the combination).  The spilling kernels stay in the object,
+    # unused; "rerouted" names them.
+    m = plan.get("mapping", {})
+    ragged = lambda names: [k for k in names if re.match(r"tc_mfma_kernel<[01],[01],1,[01]>$", k) and not k.startswith("tc_mfma_kernel<1,1,")]
+    if ragged(spilling) and m.get("split_k", 1) == 1 and m.get("one_block_ragged", 1) == 1:
+        cmd2 = [c for c in cmd]
+        if "--map" in cmd2:
+            cmd2[cmd2.index("--map") + 1] += ";ok=0"
+        else:
+            cmd2 += ["--map", m["spec"] + ";ok=0"]
+        plan = json.loads(run(cmd2))
+        m = plan.get("mapping", {})
+        remarks = run(["hipcc"] + HIPCC_FLAGS + [RESOURCE_FLAG, "-o", os.path.join(LIB, name + ".so"), hip])
+        res = kernel_resources(remarks)
+        spilling = is_spilling(res)
+    rerouted = ragged(spilling) if m.get("one_block_ragged", 1) == 0 else []
     hot = hot_kernel(plan, entry["bench_sizes"]) if "mapping" in plan else None      # (a fused group has one kernel of its own)
     with open(os.path.join(LIB, name + ".resources.json"), "w") as f:
-        json.dump({"hot": hot, "spilling": spilling, "kernels": res}, f, indent=1, sort_keys=True)
+        json.dump({"hot": hot, "spilling": spilling, "rerouted": rerouted, "kernels": res}, f, indent=1, sort_keys=True)
     bad = [k for k in spilling if hot is None or k == hot]
     if bad and not entry.get("allow_scratch"):
         raise RuntimeError("%s: the kernel for its benchmark extents spills registers to scratch memory: %s (mapping %s)"

@@ -354,7 +354,11 @@ int tc_run(const int* sizes, void* C, const void* A, const void* B, hipStream_t 
     if (variant == TC_VARIANT_AUTO && tc_stream_launch<Cfg>(ext_div, int_div, nkb, swp, stream, c, x, y, d)) {
         tc_last_kernel() = TC_KERNEL_STREAM;
     } else {
-        tc_launch_variant<Cfg>(nkb == 1, ext_full, int_full, swp, g, b, stream, c, x, y, d);
+        // (Cfg::OKP == 0: a single K block goes through the K-loop kernels, which run it as a loop of one trip, unless
+        // every tile of the call is whole; only mappings without split K may say so)
+        static_assert(Cfg::OKP != 0 || Cfg::SK == 1, "ok=0 needs a mapping without split K");
+        const bool one_kb = nkb == 1 && ((int_full && ext_full) || Cfg::OKP != 0);
+        tc_launch_variant<Cfg>(one_kb, ext_full, int_full, swp, g, b, stream, c, x, y, d);
         tc_last_kernel() = TC_KERNEL_TILED;
     }
     const int rc = tc_check_launch("tiled kernel launch failed");

@@ -105,7 +105,7 @@ void emit_cfg_members(std::ostringstream& o, const Contraction& c, DType t, cons
     operand("Y", yop, m.y_ids, m.y_tiles);
     o << "    static constexpr int WX = " << m.WX << ", WY = " << m.WY << ", TX = " << m.TX << ", TY = " << m.TY << ", NT = " << 64 * m.WX * m.WY << ";\n";
     o << "    static constexpr int MI = " << m.MI << ", SK = " << m.SK << ", SKO = " << m.SKO << ", MINW = " << m.MINW << ", LATEC = " << m.LATEC << ", NTC = " << m.NTC << ", SWAP = " << m.SWAP << ", PD = " << m.PD << ", RPX = " << m.RPX << ", RPY = " << m.RPY << ", CLDS = " << m.CLDS << ", NTO = " << m.NTO << ";\n";
-    o << "    static constexpr int STREAM = " << m.STREAM << ", SPD = " << m.SPD << ", SMW = " << m.SMW << ", SRES = " << m.SRES << ", SOV = " << m.SOV << ", SCD = " << m.SCD << ", SIL = " << m.SIL << ", TORD = " << m.TORD << ", DBUF = " << m.DBUF << ", ESL = " << m.ESL << ";\n";
+    o << "    static constexpr int STREAM = " << m.STREAM << ", SPD = " << m.SPD << ", SMW = " << m.SMW << ", SRES = " << m.SRES << ", SOV = " << m.SOV << ", SCD = " << m.SCD << ", SIL = " << m.SIL << ", TORD = " << m.TORD << ", DBUF = " << m.DBUF << ", ESL = " << m.ESL << ", OKP = " << m.OKP << ";\n";
     o << "    static constexpr int LAYX = " << m.layx << ", LDX = " << m.ldx << ", LAYY = " << m.layy << ", LDY = " << m.ldy << ";\n";
 }
 

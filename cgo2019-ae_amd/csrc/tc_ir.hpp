@@ -83,6 +83,7 @@ struct Mapping {
     int SRES = 0;                             // ... and which side's panel stays in LDS: 0 X (default), 1 Y (mapping spec sy=1)
     int SOV = 0;                              // 1 (mapping spec ov=1, streaming kernel): only the first slice of the resident panel is loaded before the first tile, the rest behind it
     int TORD = 0;                             // 1 (mapping spec to=1, per-tile kernel): workgroups take the tiles in the order of their origins in C's memory, no XCD-contiguous ranges
+    int OKP = 1;                              // 0 (mapping spec ok=0, no split K): calls whose contracted extents fit one K block take the K-loop kernels unless all their tiles are whole; the one-K-block kernel then serves whole tiles only
     int ESL = 0;                              // 1 (mapping spec es=1, per-tile kernel with the C tile through LDS): the first K block's slices are requested before the C tile is staged
     int SIL = 0;                              // 1 (mapping spec il=1, streaming kernel): the runs of the workgroups are interleaved (tile rn, rn + nruns, ..) instead of contiguous
     int SCD = 1;                              // (mapping spec cd=2, streaming kernel): C is read that many tiles ahead (1 or 2), in register tiles of its own

@@ -76,6 +76,7 @@ std::string Mapping::spec() const
     if (SOV) o << ";ov=1";
     if (TORD) o << ";to=1";
     if (ESL) o << ";es=1";
+    if (!OKP) o << ";ok=0";
     if (SIL) o << ";il=1";
     if (SCD > 1) o << ";cd=" << SCD;
     if (DBUF) o << ";db=1";
@@ -896,6 +897,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
         else if (key == "ov") m.SOV = atoi(val.c_str()) ? 1 : 0;
         else if (key == "to") m.TORD = atoi(val.c_str()) ? 1 : 0;
         else if (key == "es") m.ESL = atoi(val.c_str()) ? 1 : 0;
+        else if (key == "ok") m.OKP = atoi(val.c_str()) ? 1 : 0;
         else if (key == "il") m.SIL = atoi(val.c_str()) ? 1 : 0;
         else if (key == "cd") m.SCD = std::max(1, std::min(2, atoi(val.c_str())));
         else if (key == "rx") m.RPX = atoi(val.c_str()) ? 1 : 0;
@@ -925,6 +927,7 @@ bool mapping_from_spec(const Contraction& c, DType t, const ArchGfx950& arch, co
     if (!check_mapping(c, t, arch, m, err)) return false;
     // the streaming kernel gives every output tile to exactly one workgroup: K shares cannot be combined with it
     if (m.st_forced > 0 && m.SK > 1) { err = "mapping spec: st= (streaming kernel) and sk= (split K) exclude each other"; return false; }
+    if (!m.OKP && m.SK > 1) { err = "mapping spec: ok=0 (ragged single K blocks through the K-loop kernels) and sk= (split K) exclude each other"; return false; }
     if (m.st_forced > 0 && !plan_stream(c, t, arch, m, err)) return false;
     cost_model(c, t, arch, m);
     return true;
@@ -946,7 +949,7 @@ std::string mapping_json(const Contraction& c, DType t, const Mapping& m)
     const char* names[3] = {"v_mfma_f64_16x16x4_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"};
     o << "\"block_tile\": [" << m.BX << ", " << m.BY << ", " << m.BK << "], \"padded\": [" << m.BXP << ", " << m.BYP << ", " << m.BKP << "], "
       << "\"waves\": [" << m.WX << ", " << m.WY << "], \"mfma_tiles_per_wave\": [" << m.TX << ", " << m.TY << "], "
-      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"split_k_outermost\": " << m.SKO << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"stream_resident\": \"" << (m.SRES ? "y" : "x") << "\", \"stream_panel_overlap\": " << m.SOV << ", \"stream_c_distance\": " << m.SCD << ", \"stream_interleaved_runs\": " << m.SIL << ", \"tile_order_c_memory\": " << m.TORD << ", \"early_slices\": " << m.ESL << ", \"dynamic_lds_stages\": " << m.DBUF << ", \"vector_slice_loads\": " << m.VL << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
+      << "\"mfma\": \"" << names[m.MI] << "\", \"split_k\": " << m.SK << ", \"split_k_outermost\": " << m.SKO << ", \"min_waves_per_simd\": " << m.MINW << ", \"late_c\": " << m.LATEC << ", \"nontemporal_c\": " << m.NTC << ", \"swapped_roles\": " << m.SWAP << ", \"prefetch_depth\": " << m.PD << ", \"nontemporal_inputs\": " << m.NTO << ", \"stream\": [" << m.STREAM << ", " << m.SPD << "], \"stream_resident\": \"" << (m.SRES ? "y" : "x") << "\", \"stream_panel_overlap\": " << m.SOV << ", \"stream_c_distance\": " << m.SCD << ", \"stream_interleaved_runs\": " << m.SIL << ", \"tile_order_c_memory\": " << m.TORD << ", \"early_slices\": " << m.ESL << ", \"one_block_ragged\": " << m.OKP << ", \"dynamic_lds_stages\": " << m.DBUF << ", \"vector_slice_loads\": " << m.VL << ", \"c_through_lds\": " << m.CLDS << ", \"repack\": [" << m.RPX << ", " << m.RPY << "], \"threads\": " << 64 * m.WX * m.WY << ", "
       << "\"lds_layout\": [" << m.layx << ", " << m.layy << "], \"lds_ld\": [" << m.ldx << ", " << m.ldy << "], \"lds_bytes\": " << m.lds_bytes << ", "
       << "\"model\": {\"blocks\": " << m.n_blocks << ", \"k_steps\": " << m.steps_main_loop << ", \"blocks_per_cu\": " << m.blocks_per_cu
       << ", \"t_hbm_us\": " << m.t_hbm * 1e6 << ", \"t_l2_us\": " << m.t_l2 * 1e6 << ", \"t_mfma_us\": " << m.t_mfma * 1e6

@@ -55,6 +55,13 @@ def test_no_benchmark_kernel_spills_registers():
         assert 0 < k["vgprs"] + k.get("agprs", 0) <= 512 and k["occupancy"] >= 1
         if e["name"].startswith("cfg"):
             assert hot not in res["spilling"]
+        # Kernels for other extents that spill: the one-K-block kernels for ragged tiles are taken out of use by
+        # re-emitting the object with ok=0 ("rerouted"); nothing else may spill in a benchmark object.
+        in_use = [k for k in res["spilling"] if k not in res.get("rerouted", [])]
+        if not e["name"].startswith("var_"):
+            assert in_use == [], (e["name"], in_use)
+        if res.get("rerouted"):
+            assert ";ok=0" in cogent_mi355.Expression(e["name"]).info["spec"]
 
 
 def test_driver_library_exports():

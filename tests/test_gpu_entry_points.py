@@ -117,3 +117,27 @@ def test_entry_point_inside_a_captured_graph(tools, oracle):
         torch.cuda.synchronize()
         got = dC.cpu().numpy()
         assert helpers.rel_error(got, want2) <= 1e-12, "replay %d" % replay
+
+
+@pytest.mark.parametrize("sizes", [[24, 16, 16, 24, 1, 5],      # whole output tiles, one K block that is not full
+                                   [11, 9, 6, 10, 1, 5],        # ragged output tiles, the same
+                                   [24, 16, 16, 24, 1, 8],      # one full K block, whole tiles: the one-K-block kernel serves it
+                                   [11, 9, 6, 10, 1, 8],        # one full K block, ragged output tiles: the K loop again
+                                   [48, 8, 8, 24, 3, 7]],       # three ragged K blocks: the K loop proper
+                         ids=["full-tiles", "ragged-tiles", "full-block", "full-block-ragged-tiles", "k-loop"])
+def test_ragged_single_k_block_through_the_k_loop_kernels(sizes, tools, oracle):
+    """Mapping option ok=0: a call whose contracted extents fit one K block takes the K-loop kernels (one trip) unless
+    all its tiles are whole, instead of the one-K-block kernels, whose variants for ragged tiles spill registers on
+    this 192x192 tile.  Every element against the oracle."""
+    import cogent_mi355 as pkg
+    from gpu_common import make_inputs, run_entry
+    name = "var_tccg20_ragged_k_loop_f64"
+    ex = pkg.Expression(name)
+    assert ex.info["one_block_ragged"] == 0 and ";ok=0" in ex.info["spec"]
+    expr = helpers.parse_expression(pkg.expression_text(name))
+    print("[gpu] %s sizes=%s" % (name, sizes), flush=True)
+    C, A, B = make_inputs(tools, expr, sizes, np.float64)
+    got = run_entry(ex, sizes, C, A, B)
+    assert ex.last_kernel() == "tiled"
+    want = oracle.contract(expr, sizes, C.copy(), A, B)
+    assert helpers.rel_error(got, want) <= 1e-12

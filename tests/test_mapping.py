@@ -97,6 +97,12 @@ def test_kernel_options_in_a_spec(tools):
     m = tools.plan(text, "DOUBLE", mapping_spec=small + ";cl=1;es=1").info["mapping"]
     assert m["early_slices"] == 1 and m["spec"].endswith(";es=1")
     assert tools.plan(text, "DOUBLE", mapping_spec=m["spec"]).info["mapping"] == m
+    # ok=0: single K blocks with ragged tiles through the K-loop kernels; not with split K
+    m = tools.plan(text, "DOUBLE", mapping_spec=base + ";ok=0").info["mapping"]
+    assert m["one_block_ragged"] == 0 and m["spec"].endswith(";ok=0")
+    assert tools.plan(text, "DOUBLE", mapping_spec=base).info["mapping"]["one_block_ragged"] == 1
+    with pytest.raises(Exception, match="exclude"):
+        tools.plan(text, "DOUBLE", mapping_spec=base + ";sk=2;ok=0")
     # rx=/ry=: an input copied into tile order first; its slices then go to LDS K-major whatever its own order
     m = tools.plan(text, "DOUBLE", mapping_spec="x=d:72,c:2;y=b:24,a:2;k=e:12;w=3x1;t=3x3;rx=1;ry=1").info["mapping"]
     assert m["repack"] == [1, 1] and m["lds_layout"] == [0, 0] and "rx=1" in m["spec"] and "ry=1" in m["spec"]
